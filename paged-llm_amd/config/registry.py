@@ -32,6 +32,10 @@ def register_architecture(arch: Architecture) -> None:
 def lookup_architecture(hf_config: dict) -> Architecture:
     from .. import models  # noqa: F401  (importing the package registers the architectures it ships)
     names = hf_config.get("architectures") or []
+    if isinstance(names, str):
+        names = [names]
+    if not names and isinstance(hf_config.get("architecture"), str):        # (some families name one architecture, in the singular)
+        names = [hf_config["architecture"]]
     for n in names:
         if n in ARCHITECTURES:
             return ARCHITECTURES[n]

@@ -1,0 +1,113 @@
+// Kernels for models whose residual stream is kept in float whatever the compute type: the embedding gather
+// with a scale, a layer norm (weight and bias) of a branch's output that is added to the stream in the same
+// kernel, and the conversion of stream rows to the compute type for the next product.  All arithmetic is
+// float; T is only the storage type of the rows that go into or come out of matrix products.
+#include "common.h"
+
+using namespace pllm;
+
+// ---------------------------------------------------------------------------------------------
+// x[t, :] = float(table[ids[t], :]) * scale;  rows[t, :] = T(x[t, :]) when asked for.
+template <typename T>
+__global__ void embed_scaled_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ x,
+                                    T* __restrict__ rows, int hidden, int vocab, float scale) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range; never fault
+  const T* src = table + (size_t)id * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = to_f32(src[i]) * scale;
+    x[(size_t)t * hidden + i] = v;
+    if (rows) rows[(size_t)t * hidden + i] = from_f32<T>(v);
+  }
+}
+
+PLLM_API int pllm_embed_scaled(int dtype, const int* ids, const void* table, float* x, void* rows, int num_tokens,
+                               int hidden, int vocab, float scale, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(embed_scaled_kernel<float>, grid, block, 0, stream, ids, (const float*)table, x, (float*)rows, hidden, vocab, scale);
+  else
+    hipLaunchKernelGGL(embed_scaled_kernel<bf16>, grid, block, 0, stream, ids, (const bf16*)table, x, (bf16*)rows, hidden, vocab, scale);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Layer norm of one row per workgroup:  y = (v - mean) / sqrt(var + eps) * w + b,  var = mean((v - mean)^2),
+// with v = in[src] (src = row_index[r] or r).  Then
+//   stream given:  stream[r] += y (float), and rows[r] = T(stream[r]) when rows is given;
+//   no stream:     rows[r] = T(y).
+// TI is the type of `in` (float, or the compute type), TO the type of `rows`.
+template <typename TI, typename TO>
+__global__ void layernorm_kernel(const TI* __restrict__ in, const int* __restrict__ row_index, const float* __restrict__ w,
+                                 const float* __restrict__ b, float eps, float* stream_rows, TO* __restrict__ rows, int hidden) {
+  extern __shared__ float lds[];
+  float* row = lds;               // [hidden]
+  float* scratch = lds + hidden;  // [16]
+  const int r = blockIdx.x;
+  const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
+  const TI* v = in + src * hidden;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float f = to_f32(v[i]);
+    row[i] = f;
+    acc += f;
+  }
+  const float mean = block_sum(acc, scratch) / (float)hidden;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float d = row[i] - mean;
+    sq = fmaf(d, d, sq);
+  }
+  const float var = block_sum(sq, scratch) / (float)hidden;
+  const float inv = 1.f / sqrtf(var + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float y = (row[i] - mean) * inv * w[i] + b[i];
+    if (stream_rows) {
+      y += stream_rows[(size_t)r * hidden + i];
+      stream_rows[(size_t)r * hidden + i] = y;
+    }
+    if (rows) rows[(size_t)r * hidden + i] = from_f32<TO>(y);
+  }
+}
+
+// in_dtype / out_dtype: PLLM_F32 or PLLM_BF16.
+PLLM_API int pllm_layernorm(int in_dtype, int out_dtype, const void* in, const int* row_index, const float* w, const float* b,
+                            float eps, float* stream_rows, void* rows, int num_rows, int hidden, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  if (hidden <= 0) return -2;
+  dim3 grid(num_rows), block(256);
+  const size_t lds = (size_t)(hidden + 16) * sizeof(float);
+#define PLLM_LN(TI, TO)                                                                                                          \
+  do {                                                                                                                          \
+    if (lds > 48 * 1024) {                                                                                                      \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(layernorm_kernel<TI, TO>),                               \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                \
+      if (e != hipSuccess) return (int)e;                                                                                       \
+    }                                                                                                                           \
+    hipLaunchKernelGGL((layernorm_kernel<TI, TO>), grid, block, lds, stream, (const TI*)in, row_index, w, b, eps, stream_rows, \
+                       (TO*)rows, hidden);                                                                                      \
+  } while (0)
+  if (in_dtype == PLLM_F32 && out_dtype == PLLM_F32) PLLM_LN(float, float);
+  else if (in_dtype == PLLM_F32 && out_dtype == PLLM_BF16) PLLM_LN(float, bf16);
+  else if (in_dtype == PLLM_BF16 && out_dtype == PLLM_BF16) PLLM_LN(bf16, bf16);
+  else if (in_dtype == PLLM_BF16 && out_dtype == PLLM_F32) PLLM_LN(bf16, float);
+  else return -3;
+#undef PLLM_LN
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// rows = bf16(x), element by element.
+__global__ void round_rows_kernel(const float* __restrict__ x, bf16* __restrict__ rows, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    rows[i] = __float2bfloat16(x[i]);
+}
+
+PLLM_API int pllm_round_rows(const float* x, void* rows, long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  hipLaunchKernelGGL(round_rows_kernel, dim3(blocks), dim3(256), 0, stream, x, (bf16*)rows, (size_t)n);
+  PLLM_RETURN_LAST_ERROR();
+}

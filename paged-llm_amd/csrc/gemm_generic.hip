@@ -14,7 +14,11 @@ constexpr int BM = 64, BN = 64, BK = 16;
 
 template <typename TA, typename TC>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, int lda, const TA* __restrict__ W, int ldw,
-                                                      TC* __restrict__ C, int ldc, int M, int N, int K) {
+                                                      TC* __restrict__ C, int ldc, int M, int N, int K,
+                                                      long a_batch, long w_batch, long c_batch) {
+  A += (size_t)blockIdx.z * a_batch;          // one product per blockIdx.z (a single one: the strides are unused)
+  W += (size_t)blockIdx.z * w_batch;
+  C += (size_t)blockIdx.z * c_batch;
   __shared__ float As[BK][BM + 4];
   __shared__ float Ws[BK][BN + 4];
   const int tid = threadIdx.x;
@@ -59,22 +63,29 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
   }
 }
 
-// out_dtype may be PLLM_F32 with bf16 operands (logits).
-PLLM_API int pllm_gemm_nt(int dtype, int out_dtype, const void* A, int lda, const void* W, int ldw, void* C, int ldc,
-                          int M, int N, int K, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (K <= 0) return -2;
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM), block(256);
+// out_dtype may be PLLM_F32 with bf16 operands (logits).  `batch` products at once, operand b at its base plus b times
+// its batch stride (elements): the per-head products of a mixer, whose heads lie side by side in the rows.
+PLLM_API int pllm_gemm_nt_batched(int dtype, int out_dtype, const void* A, int lda, long a_batch, const void* W, int ldw,
+                                  long w_batch, void* C, int ldc, long c_batch, int M, int N, int K, int batch,
+                                  hipStream_t stream) {
+  if (M <= 0 || N <= 0 || batch <= 0) return 0;
+  if (K <= 0 || batch > 65535) return -2;
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, batch), block(256);
   if (dtype == PLLM_F32 && out_dtype == PLLM_F32)
     hipLaunchKernelGGL((gemm_nt_kernel<float, float>), grid, block, 0, stream, (const float*)A, lda, (const float*)W, ldw,
-                       (float*)C, ldc, M, N, K);
+                       (float*)C, ldc, M, N, K, a_batch, w_batch, c_batch);
   else if (dtype == PLLM_BF16 && out_dtype == PLLM_BF16)
     hipLaunchKernelGGL((gemm_nt_kernel<bf16, bf16>), grid, block, 0, stream, (const bf16*)A, lda, (const bf16*)W, ldw,
-                       (bf16*)C, ldc, M, N, K);
+                       (bf16*)C, ldc, M, N, K, a_batch, w_batch, c_batch);
   else if (dtype == PLLM_BF16 && out_dtype == PLLM_F32)
     hipLaunchKernelGGL((gemm_nt_kernel<bf16, float>), grid, block, 0, stream, (const bf16*)A, lda, (const bf16*)W, ldw,
-                       (float*)C, ldc, M, N, K);
+                       (float*)C, ldc, M, N, K, a_batch, w_batch, c_batch);
   else
     return -3;
   PLLM_RETURN_LAST_ERROR();
+}
+
+PLLM_API int pllm_gemm_nt(int dtype, int out_dtype, const void* A, int lda, const void* W, int ldw, void* C, int ldc,
+                          int M, int N, int K, hipStream_t stream) {
+  return pllm_gemm_nt_batched(dtype, out_dtype, A, lda, 0, W, ldw, 0, C, ldc, 0, M, N, K, 1, stream);
 }

@@ -1065,3 +1065,257 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                     "16..256 in steps of 16 and groups of at most 64 heads", bs, head_dim, num_heads, num_kv_heads)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window, terms=terms)
+
+
+# ------------------------------------------------------------------------------------------- a residual stream kept in float
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, want_rows: bool = True):
+    """(x, rows): x[t] = float(table[ids[t]]) * scale as float32 [T, hidden], and the same rounded to the table's type
+    (None for a float32 table, whose x already is the rows, or when ``want_rows`` is False)."""
+    _on_gpu(ids, table)
+    _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be contiguous int32 [T]")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, hidden]")
+    T, (V, H) = ids.numel(), table.shape
+    x = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    rows = torch.empty((T, H), dtype=table.dtype, device=table.device) if want_rows and table.dtype != torch.float32 else None
+    sig = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]
+    _check(_fn("float_stream.hip", "pllm_embed_scaled", signature=sig)(dtype_code(table.dtype), _ptr(ids), _ptr(table), _ptr(x), _ptr(rows),
+                                                                      T, H, V, c_float(scale), _stream()), "embed_scaled")
+    return x, rows
+
+
+def layernorm(v: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, stream_rows: torch.Tensor | None = None,
+              row_index: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """y = (v - mean) / sqrt(var + eps) * weight + bias over each row of ``v`` (float32 or bfloat16), in float.
+
+    With ``stream_rows`` (float32, as many rows as are normed): stream_rows += y in place, and the return value is the
+    new stream rounded to ``out_dtype`` (None when ``out_dtype`` is None).  Without it the return value is y in
+    ``out_dtype``.  ``row_index`` (int32) picks the rows of ``v`` that are normed."""
+    _on_gpu(v, weight, bias, stream_rows, row_index)
+    _need(v.dim() == 2 and v.is_contiguous(), "layernorm input must be contiguous [rows, hidden]")
+    H = v.shape[1]
+    for t, what in ((weight, "weight"), (bias, "bias")):
+        _need(t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous(), f"layer norm {what} must be float32 [{H}]")
+    _need((H + 16) * 4 <= min(_max_lds_bytes(v.device), 160 * 1024), f"the layer norm kernel stages one row in LDS: hidden size {H} is above its limit")
+    rows = v.shape[0]
+    if row_index is not None:
+        _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(), "row_index must be contiguous int32")
+        rows = row_index.numel()
+    if stream_rows is not None:
+        _need(stream_rows.dtype == torch.float32 and stream_rows.shape == (rows, H) and stream_rows.is_contiguous(),
+              f"the stream must be contiguous float32 [{rows}, {H}]")
+    else:
+        _need(out_dtype is not None, "layernorm without a stream returns rows: say their type")
+    out = torch.empty((rows, H), dtype=out_dtype, device=v.device) if out_dtype is not None else None
+    sig = [c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p]
+    _check(_fn("float_stream.hip", "pllm_layernorm", signature=sig)(
+        dtype_code(v.dtype), dtype_code(out_dtype or torch.float32), _ptr(v), _ptr(row_index), _ptr(weight), _ptr(bias), c_float(eps),
+        _ptr(stream_rows), _ptr(out), rows, H, _stream()), "layernorm")
+    return out
+
+
+def round_rows(x: torch.Tensor) -> torch.Tensor:
+    """float32 rows rounded to bfloat16 (the operand of a bfloat16 product read from a float stream)."""
+    _on_gpu(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "round_rows takes contiguous float32 rows")
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    _check(_fn("float_stream.hip", "pllm_round_rows", signature=[c_void_p, c_void_p, c_long, c_void_p])(_ptr(x), _ptr(out), x.numel(), _stream()),
+           "round_rows")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- per-head products
+def gemm_heads(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, h, :] = w[h] a[t, h, :] for a [T, heads, K] (a view into wider rows is fine: unit inner stride, any row and
+    head strides) and w [heads, N, K] contiguous; float accumulation in ascending k.  Returns [T, heads, N] contiguous."""
+    _on_gpu(a, w, out)
+    _need(a.dim() == 3 and w.dim() == 3 and a.shape[1] == w.shape[0] and a.shape[2] == w.shape[2] and a.dtype == w.dtype,
+          f"gemm_heads shapes {tuple(a.shape)} {a.dtype} x {tuple(w.shape)} {w.dtype}")
+    _need(a.stride(2) == 1 and w.is_contiguous(), "gemm_heads: unit inner stride of the rows, contiguous matrices")
+    T, heads, K = a.shape
+    N = w.shape[1]
+    if out is None:
+        out = torch.empty((T, heads, N), dtype=a.dtype, device=a.device)
+    _need(out.shape == (T, heads, N) and out.is_contiguous() and out.dtype == a.dtype, "bad output for gemm_heads")
+    sig = [c_int, c_int, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p]
+    _check(_fn("gemm_generic.hip", "pllm_gemm_nt_batched", signature=sig)(
+        dtype_code(a.dtype), dtype_code(out.dtype), _ptr(a), a.stride(0), a.stride(1), _ptr(w), K, N * K, _ptr(out), heads * N, N,
+        T, N, K, heads, _stream()), "gemm_heads")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- state of fixed size per request
+MAX_CONV_TAPS = 8
+
+
+def _check_sequences(state: torch.Tensor, state_slots, seq_starts, cu_seqlens, num_seqs: int) -> None:
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous(), "a state tensor is contiguous float32 [slots, size]")
+    for t, n, what in ((state_slots, num_seqs, "state_slots"), (seq_starts, num_seqs, "seq_starts"), (cu_seqlens, num_seqs + 1, "cu_seqlens")):
+        _need(t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous() and t.numel() == n, f"{what} must be contiguous int32 [{n}]")
+
+
+def causal_conv(rows: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor, state_offset: int,
+                state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int, max_q_len: int,
+                activation: str | None = "silu") -> torch.Tensor:
+    """Causal convolution per channel over each sequence's rows, then SiLU: rows [T, channels] (a view with unit inner
+    stride), weight float32 [channels, taps] (its last column meets the current token), bias float32 [channels].  The
+    last taps - 1 inputs of every sequence are read from and left in ``state[slot, state_offset : state_offset +
+    channels * (taps - 1)]``; a sequence with seq_starts == 0 starts from zeros.  The host guarantees slots < state.shape[0]."""
+    _on_gpu(rows, weight, bias, state, state_slots, seq_starts, cu_seqlens)
+    _need(rows.dim() == 2 and rows.stride(1) == 1, "causal_conv rows: [T, channels] with unit inner stride")
+    T, C = rows.shape
+    taps = weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.shape == (C, taps) and weight.is_contiguous() and 1 <= taps <= MAX_CONV_TAPS,
+          f"conv weight: float32 [{C}, taps <= {MAX_CONV_TAPS}]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (C,) and bias.is_contiguous()), f"conv bias: float32 [{C}]")
+    _need(activation in (None, "silu"), "causal_conv applies SiLU or nothing")
+    _check_sequences(state, state_slots, seq_starts, cu_seqlens, num_seqs)
+    _need(0 <= state_offset and state_offset + C * (taps - 1) <= state.shape[1], "the convolution's inputs do not fit the state slot")
+    out = torch.empty((T, C), dtype=rows.dtype, device=rows.device)
+    sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+           c_int, c_int, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_causal_conv", signature=sig)(
+        dtype_code(rows.dtype), _ptr(rows), rows.stride(0), _ptr(weight), _ptr(bias), state.data_ptr() + 4 * state_offset, state.stride(0),
+        _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens), _ptr(out), C, C, taps, 1 if activation else 0, num_seqs, max_q_len, _stream()),
+        "causal_conv")
+    return out
+
+
+def rotary_to_float(rows: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, heads: int, head_dim: int,
+                    rot_dims: int, interleaved: bool, scale: float = 1.0) -> torch.Tensor:
+    """float32 [T, heads, head_dim]: the heads of ``rows`` [T, >= heads * head_dim] (unit inner stride) with their first
+    ``rot_dims`` elements turned by the tables' angles at ``positions``, times ``scale``."""
+    _on_gpu(rows, positions, cos, sin)
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= heads * head_dim, "rotary_to_float rows: [T, >= heads * head_dim]")
+    T = rows.shape[0]
+    _need(positions.dtype == torch.int32 and positions.numel() == T and positions.is_contiguous(), "positions: int32 [T]")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= head_dim, f"rotated width {rot_dims} of a head of {head_dim}")
+    for t in (cos, sin):
+        _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot_dims // 2 and t.is_contiguous(),
+              f"rotary tables: float32 [positions, {rot_dims // 2}]")
+    out = torch.empty((T, heads, head_dim), dtype=torch.float32, device=rows.device)
+    sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_rotary_to_float", signature=sig)(
+        dtype_code(rows.dtype), _ptr(rows), rows.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out), T, heads, head_dim, rot_dims,
+        1 if interleaved else 0, c_float(scale), _stream()), "rotary_to_float")
+    return out
+
+
+def step_sizes(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> tuple:
+    """(dt, decay), float32 [T, heads]: dt = softplus(raw + bias), decay = exp(-exp(a_log) * dt); raw [T, heads] a view."""
+    _on_gpu(raw, bias, a_log)
+    _need(raw.dim() == 2 and raw.stride(1) == 1, "step_sizes raw: [T, heads] with unit inner stride")
+    T, H = raw.shape
+    for t in (bias, a_log):
+        _need(t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous(), f"step_sizes: float32 [{H}] per-head constants")
+    dt = torch.empty((T, H), dtype=torch.float32, device=raw.device)
+    decay = torch.empty((T, H), dtype=torch.float32, device=raw.device)
+    sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_step_sizes", signature=sig)(dtype_code(raw.dtype), _ptr(raw), raw.stride(0), _ptr(bias), _ptr(a_log),
+                                                                  _ptr(dt), _ptr(decay), T, H, _stream()), "step_sizes")
+    return dt, decay
+
+
+def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, state_offset: int,
+                      state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int,
+                      vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None) -> torch.Tensor:
+    """Per head:  S_t = decay_t S_(t-1) + k_t (vscale_t v_t)^T,   y_t = S_t^T q_t + skip v_t,   S [N, P] float32 at
+    ``state[slot, state_offset + head * N * P :]``; a sequence with seq_starts == 0 starts from S = 0.
+
+    q, k [T, key_heads, N] (views of one element type and one row stride, unit inner stride, heads side by side; head h
+    uses key head h // (heads / key_heads)), v [T, heads, P] likewise, decay float32 [T, heads] or [heads] (one number
+    per head for all tokens), vscale float32 [T, heads] or None, skip float32 [heads] or None.  Returns y float32 [T, heads * P]."""
+    _on_gpu(q, k, v, decay, state, state_slots, seq_starts, cu_seqlens, vscale, skip)
+    _need(q.dim() == 3 and q.shape == k.shape and q.dtype == k.dtype and q.stride() == k.stride() and q.stride(2) == 1
+          and q.stride(1) == q.shape[2], "recurrence q, k: [T, key_heads, N] views of one layout with the heads side by side")
+    _need(v.dim() == 3 and v.stride(2) == 1 and v.stride(1) == v.shape[2] and v.shape[0] == q.shape[0], "recurrence v: [T, heads, P], heads side by side")
+    T, KH, N = q.shape
+    H, P = v.shape[1], v.shape[2]
+    _need(H % KH == 0 and 1 <= N <= 1024, f"{H} heads over {KH} key heads, N = {N} (at most 1024)")
+    _need(decay.dtype == torch.float32 and decay.is_contiguous() and tuple(decay.shape) in ((T, H), (H,)), f"decay: float32 [{T}, {H}] or [{H}]")
+    _need(vscale is None or (vscale.dtype == torch.float32 and vscale.shape == (T, H) and vscale.is_contiguous()), f"vscale: float32 [{T}, {H}]")
+    _need(skip is None or (skip.dtype == torch.float32 and skip.shape == (H,) and skip.is_contiguous()), f"skip: float32 [{H}]")
+    _check_sequences(state, state_slots, seq_starts, cu_seqlens, num_seqs)
+    _need(0 <= state_offset and state_offset + H * N * P <= state.shape[1], "the recurrence's state does not fit the state slot")
+    out = torch.empty((T, H * P), dtype=torch.float32, device=v.device)
+    sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
+           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_linear_recurrence", signature=sig)(
+        _ptr(q), _ptr(k), dtype_code(q.dtype), q.stride(0), _ptr(v), dtype_code(v.dtype), v.stride(0), _ptr(decay), H if decay.dim() == 2 else 0,
+        _ptr(vscale), _ptr(skip), state.data_ptr() + 4 * state_offset, state.stride(0), _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens),
+        _ptr(out), num_seqs, H, KH, N, P, _stream()), "linear_recurrence")
+    return out
+
+
+def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor | None, group: int, gate_first: bool, eps: float) -> torch.Tensor:
+    """Behind a recurrence: y float32 [T, inner], gate [T, inner] (a view, unit inner stride) in the compute type, which is
+    also the result's.  ``gate_first``: u = y silu(gate), u / sqrt(mean(u^2) + eps) * weight over groups of ``group``
+    channels; else y / sqrt(mean(y^2) + eps) * silu(gate) (* weight when given)."""
+    _on_gpu(y, gate, weight)
+    _need(y.dtype == torch.float32 and y.dim() == 2 and y.is_contiguous(), "gated_group_norm y: contiguous float32 [T, inner]")
+    T, inner = y.shape
+    _need(gate.shape == (T, inner) and gate.stride(1) == 1, f"gate: [{T}, {inner}] with unit inner stride")
+    _need(group > 0 and inner % group == 0, f"{inner} channels in groups of {group}")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.shape == (inner,) and weight.is_contiguous()), f"weight: float32 [{inner}]")
+    out = torch.empty((T, inner), dtype=gate.dtype, device=y.device)
+    sig = [c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p]
+    _check(_fn("recurrent.hip", "pllm_gated_group_norm", signature=sig)(
+        dtype_code(gate.dtype), _ptr(y), _ptr(gate), gate.stride(0), _ptr(weight), _ptr(out), T, inner, group, 1 if gate_first else 0,
+        c_float(eps), _stream()), "gated_group_norm")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- attention over a latent
+MAX_LATENT_RANK, MAX_LATENT_ROT = 1024, 256
+
+
+def latent_prepare(rows: torch.Tensor, down_at: int, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, norm_weight: torch.Tensor,
+                   eps: float, slots: torch.Tensor | None, c_pages: torch.Tensor, kr_pages: torch.Tensor, heads: int, plain: int, rot: int,
+                   rank: int, interleaved: bool) -> None:
+    """In place on ``rows`` [T, width] = [heads x (plain | rot) | rank | rot]: the latent (columns down_at .. + rank) is
+    RMS-normed with ``norm_weight``, the shared key part behind it and every head's rot part are turned by the tables'
+    angles at ``positions``; latent and key part are written to the token's slot of ``c_pages`` [pages, block, rank] and
+    ``kr_pages`` [pages, block, rot] (no write for slot -1, or when ``slots`` is None)."""
+    _on_gpu(rows, positions, cos, sin, norm_weight, slots, c_pages, kr_pages)
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= down_at + rank + rot and down_at >= heads * (plain + rot),
+          "latent_prepare rows: [T, heads * (plain + rot) + rank + rot]")
+    T = rows.shape[0]
+    _need(rot > 0 and rot % 2 == 0 and rank > 0, f"rot {rot} (even), rank {rank}")
+    _need(positions.dtype == torch.int32 and positions.numel() == T and positions.is_contiguous(), "positions: int32 [T]")
+    for t in (cos, sin):
+        _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"rotary tables: float32 [positions, {rot // 2}]")
+    _need(norm_weight.dtype == torch.float32 and norm_weight.shape == (rank,) and norm_weight.is_contiguous(), f"latent norm weight: float32 [{rank}]")
+    _need(slots is None or (slots.dtype == torch.int32 and slots.numel() == T and slots.is_contiguous()), "slots: int32 [T]")
+    _need(c_pages.dtype == rows.dtype and kr_pages.dtype == rows.dtype and c_pages.is_contiguous() and kr_pages.is_contiguous()
+          and c_pages.dim() == 3 and c_pages.shape[2] == rank and kr_pages.shape == (*c_pages.shape[:2], rot),
+          "pages: [pages, block, rank] and [pages, block, rot] of the rows' type")
+    sig = [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+           c_int, c_int, c_int, c_void_p]
+    _check(_fn("latent_attention.hip", "pllm_latent_prepare", signature=sig)(
+        dtype_code(rows.dtype), _ptr(rows), rows.stride(0), down_at, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(norm_weight), c_float(eps),
+        _ptr(slots), _ptr(c_pages), _ptr(kr_pages), T, heads, plain, rot, rank, 1 if interleaved else 0, _stream()), "latent_prepare")
+
+
+def latent_attention(qa: torch.Tensor, rows: torch.Tensor, plain: int, rot: int, c_pages: torch.Tensor, kr_pages: torch.Tensor,
+                     block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, scale: float, window: int) -> torch.Tensor:
+    """softmax((qa . c_n + q_rot . kr_n) * scale) over the visible keys n (causal; the last ``window`` positions when
+    window > 0), times c_n: [T, heads, rank].  qa [T, heads, rank] contiguous; q_rot of head h at rows[:, h * (plain + rot) + plain:]."""
+    _on_gpu(qa, rows, c_pages, kr_pages, block_tables, cu_seqlens_q, seq_lens_k)
+    _need(qa.dim() == 3 and qa.is_contiguous() and rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[0] == qa.shape[0]
+          and rows.dtype == qa.dtype and c_pages.dtype == qa.dtype and kr_pages.dtype == qa.dtype, "latent_attention: operands of one type")
+    T, heads, rank = qa.shape
+    _need(rows.shape[1] >= heads * (plain + rot), "rows too narrow for the heads' rotated parts")
+    _need(rank <= MAX_LATENT_RANK and rot <= MAX_LATENT_ROT, f"latent sizes up to {MAX_LATENT_RANK} + {MAX_LATENT_ROT}")
+    _need(c_pages.dim() == 3 and c_pages.shape[2] == rank and kr_pages.shape == (*c_pages.shape[:2], rot) and c_pages.is_contiguous()
+          and kr_pages.is_contiguous(), "pages: [pages, block, rank] and [pages, block, rot]")
+    S = seq_lens_k.numel()
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.stride(1) == 1,
+          "block_tables: int32 [S, pages per sequence]")
+    _need(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.numel() == S + 1 and seq_lens_k.dtype == torch.int32, "lengths: int32")
+    out = torch.empty((T, heads, rank), dtype=qa.dtype, device=qa.device)
+    sig = [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+           c_int, c_int, c_int, c_float, c_int, c_void_p]
+    _check(_fn("latent_attention.hip", "pllm_latent_attention", signature=sig)(
+        dtype_code(qa.dtype), _ptr(qa), _ptr(rows), rows.stride(0), plain, _ptr(c_pages), _ptr(kr_pages), _ptr(out), _ptr(block_tables),
+        block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, heads, rank, rot, c_pages.shape[1], c_float(scale), window,
+        _stream()), "latent_attention")
+    return out

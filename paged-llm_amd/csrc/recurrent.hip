@@ -1,0 +1,343 @@
+// Kernels for mixers that carry a state of fixed size per request instead of a growing cache:
+//
+//   causal_conv            a short causal convolution per channel over the tokens of each sequence, whose last
+//                          taps - 1 inputs are carried from step to step in the request's state slot;
+//   conv_state_update      leaves those inputs for the next step;
+//   rotary_to_float        rotary encoding of heads into float rows (what enters a recurrence stays in float);
+//   linear_recurrence      S_t = a_t S_(t-1) + k_t (g_t v_t)^T,  y_t = S_t^T q_t + skip * v_t  per head, S [N, P] in float
+//                          in the state slot: the state-space scan (k = B, q = C, v = x, a = exp(-exp(A_log) dt), g = dt,
+//                          skip = D) and retention (a = the head's decay, g = 1, no skip) are both this recurrence;
+//   gated_group_norm       the gate and the root-mean-square norm over groups of channels behind a recurrence, in
+//                          either order.
+//
+// A batch is token-major without padding: sequence s owns rows cu_seqlens[s] .. cu_seqlens[s + 1] - 1, its state
+// sits in slot state_slots[s], and seq_starts[s] == 0 says that it starts now, from a zero state, whatever the slot
+// held.  Sequences may have no rows at all.  All arithmetic is float; T is the storage type of rows.  Every token's
+// state update is done in one fixed order, so a sequence gives the same bits however it was cut into steps.
+#include "common.h"
+
+using namespace pllm;
+
+__device__ __forceinline__ float load_as_f32(const void* p, int dtype, size_t i) {
+  return dtype == PLLM_F32 ? reinterpret_cast<const float*>(p)[i] : __bfloat162float(reinterpret_cast<const bf16*>(p)[i]);
+}
+__device__ __forceinline__ float silu_f32(float z) { return z / (1.f + expf(-z)); }
+
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxTaps = 8;
+constexpr int kConvChunk = 64;     // tokens of one sequence that one workgroup walks
+
+// out[t, c] = act(bias[c] + sum_j w[c, j] * in[t - (taps - 1) + j, c]); the last column of w meets the current token;
+// inputs before the sequence's first token of this step come from the state (or are zero for a sequence that starts).
+// state: [slots][channels][taps - 1] floats, oldest input first.
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(
+    const T* __restrict__ in, int in_stride, const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, size_t slot_stride, const int* __restrict__ state_slots,
+    const int* __restrict__ seq_starts, const int* __restrict__ cu_seqlens, T* __restrict__ out, int out_stride,
+    int channels, int taps, int act) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int seq = blockIdx.y;
+  const int q_begin = cu_seqlens[seq], q_len = cu_seqlens[seq + 1] - q_begin;
+  const int t0 = blockIdx.z * kConvChunk;
+  if (c >= channels || t0 >= q_len) return;
+  const int t1 = t0 + kConvChunk < q_len ? t0 + kConvChunk : q_len;
+  const bool carried = seq_starts[seq] > 0;
+  const float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * (taps - 1);
+  float wj[kMaxTaps], win[kMaxTaps];
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) {
+    wj[j] = j < taps ? w[(size_t)c * taps + j] : 0.f;
+    win[j] = 0.f;
+    if (j < taps - 1) {
+      const int rel = t0 - (taps - 1) + j;      // token of this step (>= 0) or an input of earlier steps (< 0)
+      if (rel >= 0) win[j] = to_f32(in[(size_t)(q_begin + rel) * in_stride + c]);
+      else if (carried) win[j] = st[(taps - 1) + rel];
+    }
+  }
+  const float b = bias ? bias[c] : 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const float cur = to_f32(in[(size_t)(q_begin + t) * in_stride + c]);
+    float acc = b;
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j < taps - 1) acc = fmaf(wj[j], win[j], acc);
+#pragma unroll
+    for (int j = 0; j < kMaxTaps; ++j)
+      if (j == taps - 1) acc = fmaf(wj[j], cur, acc);
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j) {
+      if (j < taps - 2) win[j] = win[j + 1];
+      else if (j == taps - 2) win[j] = cur;
+    }
+    out[(size_t)(q_begin + t) * out_stride + c] = from_f32<T>(act ? silu_f32(acc) : acc);
+  }
+}
+
+// state[k] <- the input at token q_len - (taps - 1) + k of this step, or what the state held for it.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    const T* __restrict__ in, int in_stride, float* state, size_t slot_stride, const int* __restrict__ state_slots,
+    const int* __restrict__ seq_starts, const int* __restrict__ cu_seqlens, int channels, int taps) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int seq = blockIdx.y;
+  if (c >= channels) return;
+  const int q_begin = cu_seqlens[seq], q_len = cu_seqlens[seq + 1] - q_begin;
+  const bool carried = seq_starts[seq] > 0;
+  float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * (taps - 1);
+  float nv[kMaxTaps];
+#pragma unroll
+  for (int k = 0; k < kMaxTaps - 1; ++k) {
+    nv[k] = 0.f;
+    if (k < taps - 1) {
+      const int rel = q_len - (taps - 1) + k;
+      if (rel >= 0) nv[k] = to_f32(in[(size_t)(q_begin + rel) * in_stride + c]);
+      else if (carried) nv[k] = st[q_len + k];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kMaxTaps - 1; ++k)
+    if (k < taps - 1) st[k] = nv[k];
+}
+
+PLLM_API int pllm_causal_conv(int dtype, const void* in, int in_stride, const float* w, const float* bias, float* state,
+                              long slot_stride, const int* state_slots, const int* seq_starts, const int* cu_seqlens,
+                              void* out, int out_stride, int channels, int taps, int act, int num_seqs, int max_q_len,
+                              hipStream_t stream) {
+  if (num_seqs <= 0 || max_q_len <= 0 || channels <= 0) return 0;
+  if (taps < 1 || taps > kMaxTaps) return -2;
+  dim3 block(256), grid((channels + 255) / 256, num_seqs, (max_q_len + kConvChunk - 1) / kConvChunk);
+  dim3 grid_state((channels + 255) / 256, num_seqs);
+  if (dtype == PLLM_F32) {
+    hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, stream, (const float*)in, in_stride, w, bias, state,
+                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (float*)out, out_stride, channels, taps, act);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<float>, grid_state, block, 0, stream, (const float*)in, in_stride, state,
+                         (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
+  } else {
+    hipLaunchKernelGGL(causal_conv_kernel<bf16>, grid, block, 0, stream, (const bf16*)in, in_stride, w, bias, state,
+                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (bf16*)out, out_stride, channels, taps, act);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<bf16>, grid_state, block, 0, stream, (const bf16*)in, in_stride, state,
+                         (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
+  }
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, h, i] = float(rotated in[t, h, i]) * scale: the first rot_dims elements of each head turn by the angle of the
+// token's position (tables cos/sin [positions, rot_dims / 2]); partners are (i, i + rot_dims / 2) or, interleaved,
+// (2i, 2i + 1).  The result stays in float.
+template <typename T>
+__global__ void rotary_to_float_kernel(const T* __restrict__ in, int in_stride, const int* __restrict__ positions,
+                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t, float* __restrict__ out,
+                                       int heads, int head_dim, int rot_dims, int interleaved, float scale) {
+  const int tok = blockIdx.x;
+  const int half = rot_dims / 2;
+  const T* row = in + (size_t)tok * in_stride;
+  const size_t table = (size_t)positions[tok] * half;
+  for (int idx = threadIdx.x; idx < heads * head_dim; idx += blockDim.x) {
+    const int h = idx / head_dim, i = idx % head_dim;
+    const T* head = row + (size_t)h * head_dim;
+    float val = to_f32(head[i]);
+    if (i < rot_dims) {
+      int pair, partner;
+      bool upper;
+      if (interleaved) { pair = i >> 1; upper = i & 1; partner = i ^ 1; }
+      else { upper = i >= half; pair = upper ? i - half : i; partner = upper ? i - half : i + half; }
+      const float other = to_f32(head[partner]);
+      float lo, hi;
+      rotate_pair(upper ? other : val, upper ? val : other, cos_t[table + pair], sin_t[table + pair], lo, hi);
+      val = upper ? hi : lo;
+    }
+    out[(size_t)tok * heads * head_dim + idx] = val * scale;
+  }
+}
+
+PLLM_API int pllm_rotary_to_float(int dtype, const void* in, int in_stride, const int* positions, const float* cos_t,
+                                  const float* sin_t, float* out, int num_tokens, int heads, int head_dim, int rot_dims,
+                                  int interleaved, float scale, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (rot_dims < 0 || rot_dims > head_dim || rot_dims % 2) return -2;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(rotary_to_float_kernel<float>, grid, block, 0, stream, (const float*)in, in_stride, positions, cos_t, sin_t,
+                       out, heads, head_dim, rot_dims, interleaved, scale);
+  else
+    hipLaunchKernelGGL(rotary_to_float_kernel<bf16>, grid, block, 0, stream, (const bf16*)in, in_stride, positions, cos_t, sin_t,
+                       out, heads, head_dim, rot_dims, interleaved, scale);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+struct RecurrenceArgs {
+  const void* q; const void* k;        // [T, key_heads, N], element type qk_dtype, row stride qk_stride (elements)
+  const void* v;                       // [T, heads, P], element type v_dtype, row stride v_stride
+  const float* decay;                  // a_t per head: decay[t * decay_stride + h] (decay_stride 0: one number per head)
+  const float* vscale;                 // g_t per head [T, heads], or null for 1
+  const float* skip;                   // [heads] or null
+  float* state;                        // slot s, head h: state + s * slot_stride + h * N * P, as [N][P]
+  const int* state_slots; const int* seq_starts; const int* cu_seqlens;
+  float* out;                          // [T, heads * P]
+  long slot_stride;
+  int qk_dtype, qk_stride, v_dtype, v_stride, decay_stride;
+  int heads, key_heads, N, P, pblocks;
+};
+
+// One workgroup per (sequence, head, block of 64 value channels); lane = value channel, so a token's update needs no
+// exchange between lanes.  Wave w holds rows w * NR .. w * NR + NR - 1 of S in registers; with several waves their
+// partial outputs are added through LDS in wave order.  A token's k and q are fetched by one lane each and read out
+// lane by lane.
+template <int NR, int MAX_THREADS>
+__global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(RecurrenceArgs a) {
+  __shared__ float part[2][MAX_THREADS / 64][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int head = blockIdx.x / a.pblocks, pb = blockIdx.x % a.pblocks;
+  const int p = pb * 64 + lane;
+  const bool p_ok = p < a.P;
+  const int seq = blockIdx.y;
+  const int q_begin = a.cu_seqlens[seq], q_len = a.cu_seqlens[seq + 1] - q_begin;
+  if (q_len <= 0) return;
+  const int kh = head / (a.heads / a.key_heads);
+  const int n0 = wv * NR;
+  const bool carried = a.seq_starts[seq] > 0;
+  float* st = a.state + (size_t)a.state_slots[seq] * a.slot_stride + (size_t)head * a.N * a.P;
+  float S[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) S[i] = (carried && p_ok && n0 + i < a.N) ? st[(size_t)(n0 + i) * a.P + p] : 0.f;
+  const float skip = a.skip ? a.skip[head] : 0.f;
+  const bool mine = lane < NR && n0 + lane < a.N;
+  for (int t = 0; t < q_len; ++t) {
+    const size_t row = (size_t)(q_begin + t);
+    const size_t qk_at = row * a.qk_stride + (size_t)kh * a.N + n0 + lane;
+    const float k_l = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
+    const float q_l = mine ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
+    const float dec = a.decay[row * a.decay_stride + head];
+    const float x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
+    const float xg = a.vscale ? x * a.vscale[row * a.heads + head] : x;
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const float kk = row_lane(k_l, i), qq = row_lane(q_l, i);
+      S[i] = fmaf(kk, xg, dec * S[i]);
+      y[i & 3] = fmaf(S[i], qq, y[i & 3]);
+    }
+    float total = (y[0] + y[1]) + (y[2] + y[3]);
+    if (waves > 1) {
+      part[t & 1][wv][lane] = total;
+      __syncthreads();
+      if (wv == 0) {
+        total = part[t & 1][0][lane];
+        for (int w = 1; w < waves; ++w) total += part[t & 1][w][lane];
+      }
+    }
+    if (wv == 0 && p_ok) a.out[row * (size_t)(a.heads * a.P) + (size_t)head * a.P + p] = fmaf(skip, x, total);
+  }
+  if (p_ok) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+      if (n0 + i < a.N) st[(size_t)(n0 + i) * a.P + p] = S[i];
+  }
+}
+
+PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, int qk_stride, const void* v, int v_dtype,
+                                    int v_stride, const float* decay, int decay_stride, const float* vscale, const float* skip,
+                                    float* state, long slot_stride, const int* state_slots, const int* seq_starts,
+                                    const int* cu_seqlens, float* out, int num_seqs, int heads, int key_heads, int N, int P,
+                                    hipStream_t stream) {
+  if (num_seqs <= 0) return 0;
+  if (heads <= 0 || key_heads <= 0 || heads % key_heads || N <= 0 || N > 1024 || P <= 0) return -2;
+  RecurrenceArgs a;
+  a.q = q; a.k = k; a.v = v; a.decay = decay; a.vscale = vscale; a.skip = skip; a.state = state;
+  a.state_slots = state_slots; a.seq_starts = seq_starts; a.cu_seqlens = cu_seqlens; a.out = out;
+  a.slot_stride = slot_stride; a.qk_dtype = qk_dtype; a.qk_stride = qk_stride; a.v_dtype = v_dtype; a.v_stride = v_stride;
+  a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = P; a.pblocks = (P + 63) / 64;
+  const int waves = (N + 63) / 64, need = (N + waves - 1) / waves;   // rows of S per wave
+  dim3 grid(heads * a.pblocks, num_seqs), block(64 * waves);
+  if (waves > 4) hipLaunchKernelGGL((linear_recurrence_kernel<64, 1024>), grid, block, 0, stream, a);
+  else if (need <= 8) hipLaunchKernelGGL((linear_recurrence_kernel<8, 256>), grid, block, 0, stream, a);
+  else if (need <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<16, 256>), grid, block, 0, stream, a);
+  else if (need <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<32, 256>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((linear_recurrence_kernel<64, 256>), grid, block, 0, stream, a);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// decay[t, h] = exp(-exp(A_log[h]) * dt),  dt[t, h] = softplus(raw[t, h] + bias[h])  (no clamp), both float.
+template <typename T>
+__global__ void step_sizes_kernel(const T* __restrict__ raw, int raw_stride, const float* __restrict__ bias,
+                                  const float* __restrict__ a_log, float* __restrict__ dt, float* __restrict__ decay,
+                                  int num_tokens, int heads) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= num_tokens * heads) return;
+  const int t = idx / heads, h = idx % heads;
+  const float z = to_f32(raw[(size_t)t * raw_stride + h]) + bias[h];
+  const float step = z > 20.f ? z : log1pf(expf(z));
+  dt[idx] = step;
+  decay[idx] = expf(-expf(a_log[h]) * step);
+}
+
+PLLM_API int pllm_step_sizes(int dtype, const void* raw, int raw_stride, const float* bias, const float* a_log, float* dt,
+                             float* decay, int num_tokens, int heads, hipStream_t stream) {
+  if (num_tokens <= 0 || heads <= 0) return 0;
+  dim3 block(256), grid((num_tokens * heads + 255) / 256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(step_sizes_kernel<float>, grid, block, 0, stream, (const float*)raw, raw_stride, bias, a_log, dt, decay, num_tokens, heads);
+  else
+    hipLaunchKernelGGL(step_sizes_kernel<bf16>, grid, block, 0, stream, (const bf16*)raw, raw_stride, bias, a_log, dt, decay, num_tokens, heads);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Behind a recurrence: y [T, inner] float, gate [T, inner] (row stride gate_stride), groups of `group` channels.
+//   gate_first:   u = y * silu(gate);  out = u / sqrt(mean_group(u^2) + eps) * w
+//   otherwise:    out = y / sqrt(mean_group(y^2) + eps) * silu(gate) [* w]
+// One workgroup per token.  With at least as many groups as waves each wave takes whole groups; else the workgroup
+// takes the groups one after the other.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
+                                                               int gate_stride, const float* __restrict__ w, T* __restrict__ out,
+                                                               int inner, int group, int gate_first, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int groups = inner / group;
+  const float* yr = y + (size_t)row * inner;
+  const T* gr = gate + (size_t)row * gate_stride;
+  T* orow = out + (size_t)row * inner;
+  const bool by_wave = groups >= waves;
+  const int first = by_wave ? wave : 0, step = by_wave ? waves : 1;
+  const int i0 = by_wave ? lane : threadIdx.x, di = by_wave ? 64 : blockDim.x;
+  for (int g = first; g < groups; g += step) {
+    const int base = g * group;
+    float ss = 0.f;
+    for (int i = i0; i < group; i += di) {
+      float u = yr[base + i];
+      if (gate_first) u *= silu_f32(to_f32(gr[base + i]));
+      ss = fmaf(u, u, ss);
+    }
+    ss = by_wave ? wave_sum(ss) : block_sum(ss, scratch);
+    const float inv = 1.f / sqrtf(ss / (float)group + eps);
+    for (int i = i0; i < group; i += di) {
+      const float s = silu_f32(to_f32(gr[base + i]));
+      float u = yr[base + i];
+      u = gate_first ? (u * s) * inv : (u * inv) * s;
+      if (w) u *= w[base + i];
+      orow[base + i] = from_f32<T>(u);
+    }
+  }
+}
+
+PLLM_API int pllm_gated_group_norm(int dtype, const float* y, const void* gate, int gate_stride, const float* w, void* out,
+                                   int num_tokens, int inner, int group, int gate_first, float eps, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (group <= 0 || inner % group) return -2;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, y, (const float*)gate, gate_stride, w, (float*)out,
+                       inner, group, gate_first, eps);
+  else
+    hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
+                       inner, group, gate_first, eps);
+  PLLM_RETURN_LAST_ERROR();
+}

@@ -68,6 +68,9 @@ class StepContext:
     # that norm adds float partial sums itself: the branch's last product may then return [ranges, rows, hidden] float
     # sums over ranges of its inner dimension instead of rows (``parts.linear.linear(..., partial_ok=...)``).
     partial_sums_ok: bool = False
+    # Set around a branch by a block that norms the branch's output in float before adding it: the branch's last product
+    # then returns float32 rows (no rounding to the compute type between the product's sums and the norm).
+    float_branch: bool = False
 
     @property
     def decode_only(self) -> bool:

@@ -7,6 +7,7 @@ import torch
 
 from ..cache.kv_cache import CacheGroup
 from ..parts import registry
+from ..parts.base import name_under, tensor_name
 from ..parts.registry import BuildEnv
 from ..parts.spec import ModelSpec, WeightSpec
 
@@ -32,11 +33,11 @@ class DecoderModel:
     # ------------------------------------------------------------------ weights
     def weight_specs(self) -> dict[str, WeightSpec]:
         s = self.spec
-        out = {f"{s.embedding_name}.{n}": w for n, w in self.embedding.weight_specs().items()}
+        out = {tensor_name(s.embedding_name, n): w for n, w in self.embedding.weight_specs().items()}
         for layer, block in zip(s.layers, self.blocks):
-            out.update({f"{layer.name}.{n}": w for n, w in block.weight_specs().items()})
-        out.update({f"{s.final_norm_name}.{n}": w for n, w in self.final_norm.weight_specs().items()})
-        out.update({f"{s.head_name}.{n}": w for n, w in self.head.weight_specs().items()})
+            out.update({tensor_name(layer.name, n): w for n, w in block.weight_specs().items()})
+        out.update({tensor_name(s.final_norm_name, n): w for n, w in self.final_norm.weight_specs().items()})
+        out.update({tensor_name(s.head_name, n): w for n, w in self.head.weight_specs().items()})
         return out
 
     def optional_weights(self) -> dict[str, tuple]:
@@ -49,11 +50,13 @@ class DecoderModel:
     def assign(self, name: str, tensor: torch.Tensor) -> None:
         s = self.spec
         for prefix, part in [(s.embedding_name, self.embedding), (s.final_norm_name, self.final_norm), (s.head_name, self.head)]:
-            if name.startswith(prefix + "."):
-                return part.assign(name[len(prefix) + 1:], tensor)
+            own = name_under(prefix, name)
+            if own is not None and own in part.weight_specs():
+                return part.assign(own, tensor)
         for layer, block in zip(s.layers, self.blocks):
-            if name.startswith(layer.name + "."):
-                return block.assign(name[len(layer.name) + 1:], tensor)
+            own = name_under(layer.name, name)
+            if own:
+                return block.assign(own, tensor)
         raise KeyError(name)
 
     def finalize(self) -> None:

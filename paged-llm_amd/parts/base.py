@@ -27,6 +27,19 @@ from .spec import WeightSpec
 BLOCK = "block"       # in the shape of a page tensor: the dimension that holds the positions of a page
 
 
+def tensor_name(prefix: str, name: str) -> str:
+    """The checkpoint name of a part's tensor: the part's prefix, a dot, the tensor's own name; a tensor whose own name
+    is empty bears the prefix itself (a norm's weight stored as "final.norm" beside its bias "final.norm.b")."""
+    return f"{prefix}.{name}" if name else prefix
+
+
+def name_under(prefix: str, full: str) -> str | None:
+    """The own name of the tensor ``full`` if it belongs under ``prefix`` ("" for the prefix itself), else None."""
+    if full == prefix:
+        return ""
+    return full[len(prefix) + 1:] if full.startswith(prefix + ".") else None
+
+
 @dataclass(frozen=True)
 class PageTensor:
     """One tensor of what a mixer keeps per token: the shape of ONE page, with ``BLOCK`` where the positions of the
@@ -249,14 +262,15 @@ class Block(Part):
         return False
 
     def weight_specs(self):
-        return {f"{self.names[role]}.{name}": spec for role, part in self.parts.items()
+        return {tensor_name(self.names[role], name): spec for role, part in self.parts.items()
                 for name, spec in part.weight_specs().items()}
 
     def assign(self, name, tensor):
-        for role, part in self.parts.items():
-            prefix = self.names[role] + "."
-            if name.startswith(prefix):
-                return part.assign(name[len(prefix):], tensor)
+        # (the longest prefix first: "norm1" must not take what belongs to a part named "norm1.x")
+        for role, part in sorted(self.parts.items(), key=lambda rp: -len(self.names[rp[0]])):
+            own = name_under(self.names[role], name)
+            if own is not None and own in part.weight_specs():
+                return part.assign(own, tensor)
         raise KeyError(name)
 
     def finalize(self):

@@ -8,6 +8,8 @@ stream's element type, which is what a plain add in that type gives.
 
 from __future__ import annotations
 
+import torch
+
 from .base import Block
 from .registry import register_block
 
@@ -36,3 +38,58 @@ class PreNormBlock(Block):
 
 
 register_block("prenorm", PreNormBlock)
+
+
+class BranchNormBlock(Block):
+    """A block that norms what its branches return, not what they read, over a residual stream kept in float:
+
+        x <- x + norm(mixer(x));   x <- x + norm(feed_forward(x))        (the second line only with a feed-forward)
+
+    The branches read the stream itself (rounded to the compute type where that is not float); each branch's last
+    product leaves float rows (``ctx.float_branch``), the norm runs in float and the sum stays in float: the stream is
+    never rounded.  The kernel that norms and adds also writes the new stream in the compute type, which is the next
+    branch's operand; it travels beside the stream in ``ctx.launch_cache`` so that the next block finds it.
+
+    params: the roles' prefixes in tensor names; ``feed_forward`` False for a layer with the mixer alone (its specs
+    then name no feed-forward roles)."""
+    ROLES = {"mixer": "mixer", "mixer_norm": "norm", "feed_forward": "feed_forward", "feed_forward_norm": "norm"}
+    _ROWS = "float_stream_rows"
+
+    def __init__(self, params: dict, env):
+        self.has_feed_forward = bool(params.get("feed_forward", True))
+        if not self.has_feed_forward:
+            self.ROLES = {"mixer": "mixer", "mixer_norm": "norm"}
+        super().__init__({k: v for k, v in params.items() if k in self.ROLES and isinstance(v, str)}, env)
+        self.dtype = env.dtype
+
+    def _rows(self, x, ctx):
+        """The stream in the compute type: what the kernel before left, or rounded now."""
+        if x.dtype == self.dtype:
+            return x
+        held = ctx.launch_cache.get(self._ROWS)
+        if held is not None and held[0] is x:
+            return held[1]
+        from ..csrc import ops
+        return ops.round_rows(x)
+
+    def _add(self, norm, x, branch, ctx, want_rows=True):
+        rows = norm.add_to(x, branch, want_rows)
+        ctx.launch_cache[self._ROWS] = (x, rows) if rows is not None else None
+
+    def forward(self, x, delta, ctx, cache, state):
+        p = self.parts
+        if delta is not None:
+            raise RuntimeError("a block over a float stream takes the stream with every sum done")
+        if x.dtype != torch.float32:
+            raise RuntimeError("this block keeps its residual stream in float32 (an embedding with float_stream)")
+        ctx.partial_sums_ok, ctx.float_branch = False, True
+        a = p["mixer"].forward(self._rows(x, ctx), ctx, cache, state)
+        self._add(p["mixer_norm"], x, a, ctx)
+        if self.has_feed_forward:
+            m = p["feed_forward"].forward(self._rows(x, ctx), ctx)
+            self._add(p["feed_forward_norm"], x, m, ctx)
+        ctx.float_branch = False
+        return x, None
+
+
+register_block("branch_norm", BranchNormBlock)

@@ -13,21 +13,32 @@ from .spec import WeightSpec
 
 
 class TokenEmbedding(Part):
+    """params: ``vocab_size``; ``scale`` (the gathered row is multiplied by it; default none); ``float_stream`` (the
+    rows leave as float32 whatever the compute type: the start of a residual stream that is summed in float); ``tensor_name`` (the table's own
+    name under the part's prefix, default "weight"; "" is the prefix itself)."""
+
     def __init__(self, params: dict, env: BuildEnv):
         self.vocab = int(params["vocab_size"])
         self.hidden = env.hidden_size
+        self.scale = float(params.get("scale") or 1.0)
+        self.float_stream = bool(params.get("float_stream", False))
+        self.tensor_name = params.get("tensor_name", "weight")
         self.dtype, self.device = env.dtype, env.device
         self.table: torch.Tensor | None = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.vocab, self.hidden), role="table")}
+        return {self.tensor_name: WeightSpec((self.vocab, self.hidden), role="table")}
 
     def assign(self, name, tensor):
-        if name != "weight":
+        if name != self.tensor_name:
             raise KeyError(name)
         self.table = tensor.to(device=self.device, dtype=self.dtype).contiguous()
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        if self.float_stream:
+            return ops.embed_scaled(ids, self.table, self.scale, want_rows=False)[0]
+        if self.scale != 1.0:
+            raise NotImplementedError("a scaled embedding leaves as a float stream (float_stream)")
         return ops.embed_gather(ids, self.table)
 
 
@@ -36,15 +47,16 @@ class LMHead(Part):
         self.vocab = int(params["vocab_size"])
         self.hidden = env.hidden_size
         self.tied = bool(params.get("tied", False))
+        self.tensor_name = params.get("tensor_name", "weight")      # the matrix's own name under the prefix ("": the prefix)
         self.dtype, self.device = env.dtype, env.device
         self.weight: torch.Tensor | None = None
         self._matrix = None
 
     def weight_specs(self):
-        return {} if self.tied else {"weight": WeightSpec((self.vocab, self.hidden))}
+        return {} if self.tied else {self.tensor_name: WeightSpec((self.vocab, self.hidden))}
 
     def assign(self, name, tensor):
-        if name != "weight" or self.tied:
+        if name != self.tensor_name or self.tied:
             raise KeyError(name)
         self.weight = tensor.to(device=self.device, dtype=self.dtype).contiguous()
 

@@ -57,6 +57,12 @@ STREAM_GATED_MAX_ROWS = 64                      # the gated product: beyond, its
 STREAM_LONG_K, STREAM_LONG_K_MAX_ROWS = 8192, 64 # from this K on a product in one range takes the streaming kernel up to so many rows
 
 
+def _operand(x):
+    """A product's rows as the kernels' choosers know them: a tensor, or a ``PendingNorm`` whose sum and norm a kernel may
+    take in; any other pending object (a norm that computes at once) gives its rows."""
+    return x if isinstance(x, (torch.Tensor, PendingNorm)) else x.rows()
+
+
 def _plain(weight) -> torch.Tensor:
     return weight.plain if isinstance(weight, Weight) else weight
 
@@ -154,6 +160,7 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     norm as its delta and that norm adds partial sums (``StepContext.partial_sums_ok``): the result may then be float
     [ranges, T, N], the sums over ranges of K.  ``bias`` (float32 [N]): added to the product's float sums, the result
     rounded once (a kernel of its own behind the product)."""
+    x = _operand(x)
     if bias is not None:
         sums = linear(x, weight, torch.float32)
         return ops.add_bias(sums, bias, out_dtype or _plain(weight).dtype)
@@ -222,6 +229,7 @@ def _tiles_gated(x, weight, rows: int) -> bool:
 def gated_linear(x, w_gate_up, activation: str = "silu") -> torch.Tensor:
     """act(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing);
     ``activation``: one of ``ops.ACTIVATIONS``."""
+    x = _operand(x)
     rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
     tiles = _tiles_gated(x, w_gate_up, rows)
     if not tiles and _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
@@ -247,6 +255,7 @@ def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_h
     ``position_encoding``: a part with ``cos``/``sin`` tables, ``rotary_dim`` and ``interleaved``, or None.
     The fused kernel pairs element i with i + d/2 over the whole head; another rotated width or pairing, and
     projections with a ``bias`` (float32, one value per row of ``w_qkv``), go through the product and the rotary kernel apart."""
+    x = _operand(x)
     write = k_pages is not None
     cos = sin = None
     rotary_dim, interleaved = 0, False                      # no position encoding: nothing turns

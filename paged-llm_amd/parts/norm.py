@@ -81,7 +81,7 @@ class PendingNorm:
 
 
 def rows_of(h) -> torch.Tensor:
-    return h.rows() if isinstance(h, PendingNorm) else h
+    return h if isinstance(h, torch.Tensor) else h.rows()
 
 
 class RMSNorm(Norm):
@@ -113,3 +113,48 @@ class RMSNorm(Norm):
 
 
 register_norm("rmsnorm", RMSNorm)
+
+
+class LayerNorm(Norm):
+    """Layer norm with weight and bias, y = (v - mean) / sqrt(var + eps) * w + b with var the mean of the squared
+    deviations, computed in float whatever the compute type.  Two uses: ``forward`` norms rows of a stream (the last
+    norm in front of the head) and ``add_to`` norms a branch's output and adds it to a float residual stream in the same
+    kernel (a block that norms what its branches return, not what they read).
+
+    params: ``eps``; ``size`` (default: the model's width); ``weight_name`` / ``bias_name``: the tensors' own names
+    under the part's prefix (defaults "weight" and "bias"; "" is the prefix itself)."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.eps = float(params["eps"])
+        self.size = int(params.get("size", env.hidden_size))
+        self.weight_name = params.get("weight_name", "weight")
+        self.bias_name = params.get("bias_name", "bias")
+        self.dtype, self.device = env.dtype, env.device
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+
+    def weight_specs(self):
+        return {self.weight_name: WeightSpec((self.size,), role="vector", init="ones"),
+                self.bias_name: WeightSpec((self.size,), role="vector", init="normal")}
+
+    def assign(self, name, tensor):
+        t = tensor.to(device=self.device, dtype=torch.float32).contiguous()
+        if name == self.weight_name:
+            self.weight = t
+        elif name == self.bias_name:
+            self.bias = t
+        else:
+            raise KeyError(name)
+
+    def forward(self, x, row_index=None):
+        """The normed rows in the compute type (x: float or compute-type rows)."""
+        return ops.layernorm(x, self.weight, self.bias, self.eps, None, row_index, self.dtype)
+
+    def add_to(self, stream: torch.Tensor, branch: torch.Tensor, want_rows: bool = True):
+        """stream += norm(branch), in place and in float; returns the new stream rounded to the compute type when that
+        is another type than the stream's and ``want_rows`` (the next product's operand), else None."""
+        out_dtype = self.dtype if want_rows and self.dtype != stream.dtype else None
+        return ops.layernorm(branch, self.weight, self.bias, self.eps, stream, None, out_dtype)
+
+
+register_norm("layernorm", LayerNorm)

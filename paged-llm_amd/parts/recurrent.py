@@ -1,0 +1,145 @@
+"""Mixers that carry a state of fixed size per request instead of a growing cache.
+
+Both are the same recurrence per head, S_t = a_t S_(t-1) + k_t (g_t v_t)^T, y_t = S_t^T q_t (+ skip v_t), with S
+[N, P] in float in the request's state slot (``ops.linear_recurrence``); they differ in where a, g, k, q and v come from:
+
+* ``mamba2`` (the state-space layer in its dual form): one input product gives a gate z, the values x, the keys B and
+  queries C of a few groups that the heads share, and a step size per head; x, B and C pass a short causal convolution
+  (whose last inputs are state too) and SiLU; a_t = exp(-exp(A_log) dt_t), g_t = dt_t = softplus(raw + bias), skip = D.
+  Behind the recurrence: times silu(z), RMS norm over parts of the channels with a weight, the output product.
+* ``retention``: q, k, v and a gate from one product, rotary encoding of q and k (kept in float), k scaled by
+  N^(-1/2), a constant decay per head; behind it each head's output divided by its root mean square, times
+  silu(gate), the output product.
+
+What enters the recurrence (step sizes, decays, rotated keys and queries, the state) is float whatever the compute type;
+the products, the convolution and the activations run in the compute type.  A request's state is zero at its first
+token (``ctx.seq_starts == 0``), whatever its slot held before.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..csrc import ops
+from .base import Mixer, StateSpec
+from .linear import Weight, linear
+from .registry import BuildEnv, register_mixer
+from .spec import PartSpec, WeightSpec
+
+
+def _out_dtype(ctx):
+    return torch.float32 if getattr(ctx, "float_branch", False) else None
+
+
+class _StatefulMixer(Mixer):
+    graph_capturable = True
+    graph_capturable_prompts = True
+    MATRICES: tuple = ()
+
+    def _keep(self, name, tensor):
+        spec = self.weight_specs().get(name)
+        if spec is None:
+            raise KeyError(name)
+        self._w[name] = tensor.to(device=self.device, dtype=torch.float32 if spec.role == "vector" else self.dtype).contiguous()
+
+    def assign(self, name, tensor):
+        self._keep(name, tensor)
+
+
+class Mamba2Mixer(_StatefulMixer):
+    """params: ``heads``, ``head_dim`` (P), ``state`` (N), ``groups``, ``conv`` (taps), ``norm_groups``, ``eps``.
+    Tensors: ``in`` [2 inner + 2 groups N + heads, width] laid out [z | x | B | C | dt], ``conv`` [inner + 2 groups N,
+    taps] with ``conv.b``, ``dt_bias``, ``A_log``, ``D`` [heads], ``norm`` [inner], ``o`` [width, inner]."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.heads, self.P, self.N = int(params["heads"]), int(params["head_dim"]), int(params["state"])
+        self.groups, self.taps = int(params.get("groups", 1)), int(params["conv"])
+        self.norm_groups, self.eps = int(params.get("norm_groups", 1)), float(params["eps"])
+        self.inner = self.heads * self.P
+        self.channels = self.inner + 2 * self.groups * self.N
+        if self.heads % self.groups or self.inner % self.norm_groups:
+            raise ValueError(f"{self.heads} heads in {self.groups} groups, {self.inner} channels normed in {self.norm_groups} parts")
+        if not 1 <= self.taps <= ops.MAX_CONV_TAPS:
+            raise ValueError(f"the convolution kernel takes 1 to {ops.MAX_CONV_TAPS} taps, got {self.taps}")
+        self.dtype, self.device = env.dtype, env.device
+        self.conv_at = self.heads * self.N * self.P              # the convolution's inputs lie behind S in the slot
+        self._w: dict = {}
+        self.w_in = self.w_o = None
+
+    def weight_specs(self):
+        H = self.heads
+        return {"in": WeightSpec((2 * self.inner + 2 * self.groups * self.N + H, self.hidden)),
+                "conv": WeightSpec((self.channels, self.taps), role="vector"), "conv.b": WeightSpec((self.channels,), role="vector"),
+                "dt_bias": WeightSpec((H,), role="vector"), "A_log": WeightSpec((H,), role="vector"), "D": WeightSpec((H,), role="vector"),
+                "norm": WeightSpec((self.inner,), role="vector", init="ones"), "o": WeightSpec((self.hidden, self.inner))}
+
+    def finalize(self):
+        self.w_in, self.w_o = Weight(self._w.pop("in")), Weight(self._w.pop("o"))
+
+    def state_spec(self):
+        return StateSpec((self.conv_at + self.channels * (self.taps - 1),), torch.float32)
+
+    def forward(self, h, ctx, cache, state):
+        w, inner, gn = self._w, self.inner, self.groups * self.N
+        proj = linear(h, self.w_in)
+        z, xbc, dt_raw = proj[:, :inner], proj[:, inner:inner + self.channels], proj[:, inner + self.channels:]
+        seqs = (ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs)
+        conv = ops.causal_conv(xbc, w["conv"], w["conv.b"], state, self.conv_at, *seqs, ctx.max_q_len)
+        dt, decay = ops.step_sizes(dt_raw, w["dt_bias"], w["A_log"])
+        x = conv[:, :inner].unflatten(1, (self.heads, self.P))
+        B = conv[:, inner:inner + gn].unflatten(1, (self.groups, self.N))
+        C = conv[:, inner + gn:].unflatten(1, (self.groups, self.N))
+        y = ops.linear_recurrence(C, B, x, decay, state, 0, *seqs, vscale=dt, skip=w["D"])
+        u = ops.gated_group_norm(y, z, w["norm"], inner // self.norm_groups, True, self.eps)
+        return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
+
+
+class RetentionMixer(_StatefulMixer):
+    """params: ``heads``, ``key_dim`` (N), ``head_dim`` (P), ``decay`` (one number per head), ``position`` (a position
+    encoding spec, or None), ``eps``.  Tensors ``q``, ``k`` [heads N, width], ``v``, ``g`` [heads P, width], ``o``."""
+
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.heads, self.N, self.P = int(params["heads"]), int(params["key_dim"]), int(params["head_dim"])
+        self.eps = float(params["eps"])
+        decay = [float(d) for d in params["decay"]]
+        if len(decay) != self.heads:
+            raise ValueError(f"{len(decay)} decays for {self.heads} heads")
+        pos = params.get("position")
+        self.position = env.position_encoding(PartSpec(**pos) if isinstance(pos, dict) else pos) if pos else None
+        self.dtype, self.device = env.dtype, env.device
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=self.device)
+        self._w: dict = {}
+        self.w_in = self.w_o = None
+
+    def weight_specs(self):
+        qk, vg = self.heads * self.N, self.heads * self.P
+        return {"q": WeightSpec((qk, self.hidden)), "k": WeightSpec((qk, self.hidden)), "v": WeightSpec((vg, self.hidden)),
+                "g": WeightSpec((vg, self.hidden)), "o": WeightSpec((self.hidden, vg))}
+
+    def finalize(self):
+        self.w_in = Weight(torch.cat([self._w.pop(n) for n in ("q", "k", "v", "g")], dim=0).contiguous())
+        self.w_o = Weight(self._w.pop("o"))
+
+    def state_spec(self):
+        return StateSpec((self.heads * self.N * self.P,), torch.float32)
+
+    def forward(self, h, ctx, cache, state):
+        H, N, P = self.heads, self.N, self.P
+        rows = linear(h, self.w_in)
+        pe = self.position
+        rot = (pe.rotary_dim or N) if pe is not None else 0
+        tables = (pe.cos, pe.sin) if pe is not None else (ctx.positions.new_zeros((1, 0), dtype=torch.float32),) * 2
+        inter = bool(pe.interleaved) if pe is not None else False
+        q = ops.rotary_to_float(rows[:, :H * N], ctx.positions, *tables, H, N, rot, inter, 1.0)
+        k = ops.rotary_to_float(rows[:, H * N:2 * H * N], ctx.positions, *tables, H, N, rot, inter, N ** -0.5)
+        v = rows[:, 2 * H * N:2 * H * N + H * P].unflatten(1, (H, P))
+        gate = rows[:, 2 * H * N + H * P:]
+        y = ops.linear_recurrence(q, k, v, self.decay, state, 0, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs)
+        u = ops.gated_group_norm(y, gate, None, P, False, self.eps)
+        return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
+
+
+register_mixer("mamba2", Mamba2Mixer)
+register_mixer("retention", RetentionMixer)
