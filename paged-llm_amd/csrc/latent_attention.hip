@@ -5,31 +5,41 @@
 // qa = W_uk^T q_plain (the query carried into the latent space) the score is (qa . c + q_rot . kr) * scale and the
 // output is W_uv (sum_n p_n c_n): the kernels here work on c and kr alone.
 //
-//   latent_prepare    per token: the RMS norm of the latent, the rotation of kr and of every head's q_rot (in place),
-//                     and the write of c and kr into the token's slot of the pages;
-//   latent_attention  one wavefront per (token, head): softmax over the visible keys (causal, and inside the window
-//                     when there is one), keys walked in tiles of 64 aligned to absolute positions, so that the order
-//                     of every sum is the same however the tokens were cut into steps or batched.
+// That is attention with one key/value head that all query heads share: key row [c | kr] (padded with zeros to
+// `width` elements), value c.  The pages hold exactly that, in the layouts of the framework's paged attention kernels,
+// which then serve this mixer as they are:
+//   k_pages [pages, 1, block_size, width]   rows [c | kr | 0]
+//   v_pages [pages, 1, width, block_size]   c transposed inside the page (optional: only for those kernels)
+// a slot is page * block_size + offset, -1 for a token that writes nothing.
 //
-//   c_pages [pages, block_size, rank], kr_pages [pages, block_size, rot]; a slot is page * block_size + offset,
-//   -1 for a token that writes nothing.  All arithmetic is float; T is the storage type.
+//   latent_prepare    per token: the RMS norm of the latent, the rotation of kr and of every head's q_rot, the write
+//                     of [c | kr] (and of c transposed) into the token's slot, and the heads' rotated query parts put
+//                     behind where their latent-space parts go in the query rows [T, heads, width];
+//   latent_attention  for latents wider than those kernels take: one wavefront per (token, head), softmax over the
+//                     visible keys (causal, inside the window when there is one), keys walked in tiles of 64 aligned
+//                     to absolute positions, so that the order of every sum is the same however the tokens were cut.
+// All arithmetic is float; T is the storage type.
 #include "common.h"
 
 using namespace pllm;
 
 // rows [T, row_stride]: heads x [plain | rot] of the queries at column 0, then the down-projection [rank | rot] at
-// column `down_at`.  The normed latent is also left in the row (in place), the rotated parts as well.
+// column `down_at`.  q_out [T, heads, width]: columns rank .. rank + rot of every head receive its rotated part and the
+// columns behind them zeros (columns 0 .. rank are another kernel's).
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(
-    T* __restrict__ rows, int row_stride, int down_at, const int* __restrict__ positions, const float* __restrict__ cos_t,
+    const T* __restrict__ rows, int row_stride, int down_at, const int* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const float* __restrict__ norm_w, float eps, const int* __restrict__ slots,
-    T* __restrict__ c_pages, T* __restrict__ kr_pages, int heads, int plain, int rot, int rank, int interleaved) {
+    T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out, int heads, int plain, int rot, int rank,
+    int width, int block_size, int interleaved) {
   __shared__ float scratch[16];
   const int tok = blockIdx.x;
-  T* row = rows + (size_t)tok * row_stride;
+  const T* row = rows + (size_t)tok * row_stride;
   const int half = rot / 2;
   const size_t table = (size_t)positions[tok] * half;
   const int slot = slots ? slots[tok] : -1;
+  T* k_row = k_pages + (size_t)(slot < 0 ? 0 : slot) * width;
+  T* v_col = v_pages ? v_pages + ((size_t)(slot < 0 ? 0 : slot / block_size) * width) * block_size + (slot < 0 ? 0 : slot % block_size) : nullptr;
   // the latent: c = down[:rank] / sqrt(mean(down[:rank]^2) + eps) * w
   float ss = 0.f;
   for (int i = threadIdx.x; i < rank; i += blockDim.x) {
@@ -37,55 +47,58 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     ss = fmaf(v, v, ss);
   }
   const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)rank + eps);
-  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
-    const T c = from_f32<T>(to_f32(row[down_at + i]) * inv * norm_w[i]);
-    row[down_at + i] = c;
-    if (slot >= 0) c_pages[(size_t)slot * rank + i] = c;
+  if (slot >= 0) {
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+      const T c = from_f32<T>(to_f32(row[down_at + i]) * inv * norm_w[i]);
+      k_row[i] = c;
+      if (v_col) v_col[(size_t)i * block_size] = c;
+    }
   }
-  // rotated parts: pair j of the shared key part (unit heads) and of every head's query part
+  // rotated parts: pair j of the shared key part (unit == heads) and of every head's query part
   for (int idx = threadIdx.x; idx < (heads + 1) * half; idx += blockDim.x) {
     const int unit = idx / half, j = idx % half;
-    T* part = unit == heads ? row + down_at + rank : row + (size_t)unit * (plain + rot) + plain;
+    const T* part = unit == heads ? row + down_at + rank : row + (size_t)unit * (plain + rot) + plain;
     const int lo_at = interleaved ? 2 * j : j, hi_at = interleaved ? 2 * j + 1 : j + half;
     float lo, hi;
     rotate_pair(to_f32(part[lo_at]), to_f32(part[hi_at]), cos_t[table + j], sin_t[table + j], lo, hi);
-    const T lo_t = from_f32<T>(lo), hi_t = from_f32<T>(hi);
-    part[lo_at] = lo_t;
-    part[hi_at] = hi_t;
-    if (unit == heads && slot >= 0) {
-      kr_pages[(size_t)slot * rot + lo_at] = lo_t;
-      kr_pages[(size_t)slot * rot + hi_at] = hi_t;
+    T* dst = unit == heads ? (slot >= 0 ? k_row + rank : nullptr) : q_out + ((size_t)tok * heads + unit) * width + rank;
+    if (dst) {
+      dst[lo_at] = from_f32<T>(lo);
+      dst[hi_at] = from_f32<T>(hi);
     }
   }
+  const int pad = width - rank - rot;
+  for (int idx = threadIdx.x; idx < heads * pad; idx += blockDim.x)
+    q_out[((size_t)tok * heads + idx / pad) * width + rank + rot + idx % pad] = from_f32<T>(0.f);
 }
 
-PLLM_API int pllm_latent_prepare(int dtype, void* rows, int row_stride, int down_at, const int* positions, const float* cos_t,
-                                 const float* sin_t, const float* norm_w, float eps, const int* slots, void* c_pages,
-                                 void* kr_pages, int num_tokens, int heads, int plain, int rot, int rank, int interleaved,
-                                 hipStream_t stream) {
+PLLM_API int pllm_latent_prepare(int dtype, const void* rows, int row_stride, int down_at, const int* positions, const float* cos_t,
+                                 const float* sin_t, const float* norm_w, float eps, const int* slots, void* k_pages,
+                                 void* v_pages, void* q_out, int num_tokens, int heads, int plain, int rot, int rank, int width,
+                                 int block_size, int interleaved, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
-  if (rot <= 0 || rot % 2 || rank <= 0 || heads <= 0 || plain < 0) return -2;
+  if (rot <= 0 || rot % 2 || rank <= 0 || heads <= 0 || plain < 0 || width < rank + rot || block_size <= 0) return -2;
   dim3 grid(num_tokens), block(256);
   if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(latent_prepare_kernel<float>, grid, block, 0, stream, (float*)rows, row_stride, down_at, positions, cos_t,
-                       sin_t, norm_w, eps, slots, (float*)c_pages, (float*)kr_pages, heads, plain, rot, rank, interleaved);
+    hipLaunchKernelGGL(latent_prepare_kernel<float>, grid, block, 0, stream, (const float*)rows, row_stride, down_at, positions, cos_t,
+                       sin_t, norm_w, eps, slots, (float*)k_pages, (float*)v_pages, (float*)q_out, heads, plain, rot, rank, width,
+                       block_size, interleaved);
   else
-    hipLaunchKernelGGL(latent_prepare_kernel<bf16>, grid, block, 0, stream, (bf16*)rows, row_stride, down_at, positions, cos_t,
-                       sin_t, norm_w, eps, slots, (bf16*)c_pages, (bf16*)kr_pages, heads, plain, rot, rank, interleaved);
+    hipLaunchKernelGGL(latent_prepare_kernel<bf16>, grid, block, 0, stream, (const bf16*)rows, row_stride, down_at, positions, cos_t,
+                       sin_t, norm_w, eps, slots, (bf16*)k_pages, (bf16*)v_pages, (bf16*)q_out, heads, plain, rot, rank, width,
+                       block_size, interleaved);
   PLLM_RETURN_LAST_ERROR();
 }
 
 constexpr int kMaxRank = 1024;      // latent sizes the attention kernel takes (16 output channels per lane)
 constexpr int kMaxRot = 256;
 
-// qa [T, heads, rank] (contiguous); q_rot of head h at rows[t * row_stride + h * (plain + rot) + plain];
-// out [T, heads, rank]: sum_n p_n c_n.
+// q [T, heads, width] rows [qa | q_rot | 0] (contiguous); out [T, heads, rank]: sum_n p_n c_n.
 template <typename T>
 __global__ __launch_bounds__(64) void latent_attention_kernel(
-    const T* __restrict__ qa, const T* __restrict__ rows, int row_stride, int plain, const T* __restrict__ c_pages,
-    const T* __restrict__ kr_pages, T* __restrict__ out, const int* __restrict__ block_tables, int bt_stride,
-    const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_seqs, int heads, int rank, int rot,
-    int block_size, float scale, int window) {
+    const T* __restrict__ q, const T* __restrict__ k_pages, T* __restrict__ out, const int* __restrict__ block_tables,
+    int bt_stride, const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_seqs, int heads,
+    int rank, int rot, int width, int block_size, float scale, int window) {
   __shared__ float q_s[kMaxRank + kMaxRot];
   __shared__ float p_s[64];
   __shared__ int slot_s[64];
@@ -103,9 +116,7 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
   const int q_pos = len_k - num_q + (tok - q_begin);
   const int* bt = block_tables + (size_t)seq * bt_stride;
 
-  for (int i = lane; i < rank; i += 64) q_s[i] = to_f32(qa[((size_t)tok * heads + head) * rank + i]);
-  for (int i = lane; i < rot; i += 64)
-    q_s[rank + i] = to_f32(rows[(size_t)tok * row_stride + (size_t)head * (plain + rot) + plain + i]);
+  for (int i = lane; i < rank + rot; i += 64) q_s[i] = to_f32(q[((size_t)tok * heads + head) * width + i]);
   __syncthreads();
 
   const int first_key = (window > 0 && q_pos - window + 1 > 0) ? q_pos - window + 1 : 0;
@@ -122,11 +133,9 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
     int slot = 0;
     if (visible) {
       slot = bt[n / block_size] * block_size + n % block_size;
-      const T* c = c_pages + (size_t)slot * rank;
-      const T* kr = kr_pages + (size_t)slot * rot;
+      const T* key = k_pages + (size_t)slot * width;
       float dot = 0.f;
-      for (int i = 0; i < rank; ++i) dot = fmaf(q_s[i], to_f32(c[i]), dot);
-      for (int i = 0; i < rot; ++i) dot = fmaf(q_s[rank + i], to_f32(kr[i]), dot);
+      for (int i = 0; i < rank + rot; ++i) dot = fmaf(q_s[i], to_f32(key[i]), dot);
       s = dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));   // finite: the tile holds at least one visible key
@@ -146,7 +155,7 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
       float a = acc[r] * alpha;
       for (int j = 0; j < count; ++j) {
         const float pj = p_s[j];
-        if (pj != 0.f) a = fmaf(pj, to_f32(c_pages[(size_t)slot_s[j] * rank + i]), a);
+        if (pj != 0.f) a = fmaf(pj, to_f32(k_pages[(size_t)slot_s[j] * width + i]), a);
       }
       acc[r] = a;
     }
@@ -159,20 +168,18 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
   }
 }
 
-PLLM_API int pllm_latent_attention(int dtype, const void* qa, const void* rows, int row_stride, int plain, const void* c_pages,
-                                   const void* kr_pages, void* out, const int* block_tables, int bt_stride,
-                                   const int* cu_seqlens_q, const int* seq_lens_k, int num_seqs, int total_q, int heads,
-                                   int rank, int rot, int block_size, float scale, int window, hipStream_t stream) {
+PLLM_API int pllm_latent_attention(int dtype, const void* q, const void* k_pages, void* out, const int* block_tables,
+                                   int bt_stride, const int* cu_seqlens_q, const int* seq_lens_k, int num_seqs, int total_q,
+                                   int heads, int rank, int rot, int width, int block_size, float scale, int window,
+                                   hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
-  if (rank <= 0 || rank > kMaxRank || rot < 0 || rot > kMaxRot || heads <= 0 || block_size <= 0) return -2;
+  if (rank <= 0 || rank > kMaxRank || rot < 0 || rot > kMaxRot || heads <= 0 || block_size <= 0 || width < rank + rot) return -2;
   dim3 grid(total_q, heads), block(64);
   if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(latent_attention_kernel<float>, grid, block, 0, stream, (const float*)qa, (const float*)rows, row_stride,
-                       plain, (const float*)c_pages, (const float*)kr_pages, (float*)out, block_tables, bt_stride, cu_seqlens_q,
-                       seq_lens_k, num_seqs, heads, rank, rot, block_size, scale, window);
+    hipLaunchKernelGGL(latent_attention_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_pages, (float*)out,
+                       block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_seqs, heads, rank, rot, width, block_size, scale, window);
   else
-    hipLaunchKernelGGL(latent_attention_kernel<bf16>, grid, block, 0, stream, (const bf16*)qa, (const bf16*)rows, row_stride,
-                       plain, (const bf16*)c_pages, (const bf16*)kr_pages, (bf16*)out, block_tables, bt_stride, cu_seqlens_q,
-                       seq_lens_k, num_seqs, heads, rank, rot, block_size, scale, window);
+    hipLaunchKernelGGL(latent_attention_kernel<bf16>, grid, block, 0, stream, (const bf16*)q, (const bf16*)k_pages, (bf16*)out,
+                       block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_seqs, heads, rank, rot, width, block_size, scale, window);
   PLLM_RETURN_LAST_ERROR();
 }

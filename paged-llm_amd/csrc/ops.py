@@ -1126,7 +1126,8 @@ def round_rows(x: torch.Tensor) -> torch.Tensor:
 # ------------------------------------------------------------------------------------------- per-head products
 def gemm_heads(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """out[t, h, :] = w[h] a[t, h, :] for a [T, heads, K] (a view into wider rows is fine: unit inner stride, any row and
-    head strides) and w [heads, N, K] contiguous; float accumulation in ascending k.  Returns [T, heads, N] contiguous."""
+    head strides) and w [heads, N, K] contiguous; float accumulation in ascending k.  Returns [T, heads, N], contiguous
+    unless ``out`` (a view of the same freedom) is given."""
     _on_gpu(a, w, out)
     _need(a.dim() == 3 and w.dim() == 3 and a.shape[1] == w.shape[0] and a.shape[2] == w.shape[2] and a.dtype == w.dtype,
           f"gemm_heads shapes {tuple(a.shape)} {a.dtype} x {tuple(w.shape)} {w.dtype}")
@@ -1135,10 +1136,10 @@ def gemm_heads(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None
     N = w.shape[1]
     if out is None:
         out = torch.empty((T, heads, N), dtype=a.dtype, device=a.device)
-    _need(out.shape == (T, heads, N) and out.is_contiguous() and out.dtype == a.dtype, "bad output for gemm_heads")
+    _need(out.shape == (T, heads, N) and out.stride(2) == 1 and out.dtype == a.dtype, "bad output for gemm_heads")
     sig = [c_int, c_int, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p]
     _check(_fn("gemm_generic.hip", "pllm_gemm_nt_batched", signature=sig)(
-        dtype_code(a.dtype), dtype_code(out.dtype), _ptr(a), a.stride(0), a.stride(1), _ptr(w), K, N * K, _ptr(out), heads * N, N,
+        dtype_code(a.dtype), dtype_code(out.dtype), _ptr(a), a.stride(0), a.stride(1), _ptr(w), K, N * K, _ptr(out), out.stride(0), out.stride(1),
         T, N, K, heads, _stream()), "gemm_heads")
     return out
 
@@ -1269,13 +1270,15 @@ MAX_LATENT_RANK, MAX_LATENT_ROT = 1024, 256
 
 
 def latent_prepare(rows: torch.Tensor, down_at: int, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, norm_weight: torch.Tensor,
-                   eps: float, slots: torch.Tensor | None, c_pages: torch.Tensor, kr_pages: torch.Tensor, heads: int, plain: int, rot: int,
-                   rank: int, interleaved: bool) -> None:
-    """In place on ``rows`` [T, width] = [heads x (plain | rot) | rank | rot]: the latent (columns down_at .. + rank) is
-    RMS-normed with ``norm_weight``, the shared key part behind it and every head's rot part are turned by the tables'
-    angles at ``positions``; latent and key part are written to the token's slot of ``c_pages`` [pages, block, rank] and
-    ``kr_pages`` [pages, block, rot] (no write for slot -1, or when ``slots`` is None)."""
-    _on_gpu(rows, positions, cos, sin, norm_weight, slots, c_pages, kr_pages)
+                   eps: float, slots: torch.Tensor | None, k_pages: torch.Tensor, v_pages: torch.Tensor | None, q_out: torch.Tensor,
+                   heads: int, plain: int, rot: int, rank: int, interleaved: bool) -> None:
+    """From ``rows`` [T, heads x (plain | rot) | rank | rot] (the down-projection at column ``down_at``): the latent
+    c = rms_norm(rows[down_at : down_at + rank]) * norm_weight and the key part behind it, turned by the tables' angles at
+    ``positions``, go to the token's slot of ``k_pages`` [pages, 1, block, width] as the row [c | key part | 0], and c
+    also to ``v_pages`` [pages, 1, width, block] (transposed inside the page) when given; no write for slot -1 or when
+    ``slots`` is None.  Every head's rotated rot part goes to ``q_out`` [T, heads, width] at columns rank .. rank + rot,
+    zeros behind it (columns 0 .. rank are left alone: the query's latent-space part belongs there)."""
+    _on_gpu(rows, positions, cos, sin, norm_weight, slots, k_pages, v_pages, q_out)
     _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= down_at + rank + rot and down_at >= heads * (plain + rot),
           "latent_prepare rows: [T, heads * (plain + rot) + rank + rot]")
     T = rows.shape[0]
@@ -1285,37 +1288,38 @@ def latent_prepare(rows: torch.Tensor, down_at: int, positions: torch.Tensor, co
         _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"rotary tables: float32 [positions, {rot // 2}]")
     _need(norm_weight.dtype == torch.float32 and norm_weight.shape == (rank,) and norm_weight.is_contiguous(), f"latent norm weight: float32 [{rank}]")
     _need(slots is None or (slots.dtype == torch.int32 and slots.numel() == T and slots.is_contiguous()), "slots: int32 [T]")
-    _need(c_pages.dtype == rows.dtype and kr_pages.dtype == rows.dtype and c_pages.is_contiguous() and kr_pages.is_contiguous()
-          and c_pages.dim() == 3 and c_pages.shape[2] == rank and kr_pages.shape == (*c_pages.shape[:2], rot),
-          "pages: [pages, block, rank] and [pages, block, rot] of the rows' type")
-    sig = [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-           c_int, c_int, c_int, c_void_p]
+    _need(k_pages.dim() == 4 and k_pages.shape[1] == 1 and k_pages.is_contiguous() and k_pages.dtype == rows.dtype, "k_pages: [pages, 1, block, width]")
+    pages, _, bs, width = k_pages.shape
+    _need(width >= rank + rot, f"pages of width {width} for a latent of {rank} + {rot}")
+    _need(v_pages is None or (v_pages.shape == (pages, 1, width, bs) and v_pages.is_contiguous() and v_pages.dtype == rows.dtype),
+          f"v_pages: [{pages}, 1, {width}, {bs}]")
+    _need(q_out.shape == (T, heads, width) and q_out.is_contiguous() and q_out.dtype == rows.dtype, f"q_out: contiguous [{T}, {heads}, {width}]")
+    sig = [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
     _check(_fn("latent_attention.hip", "pllm_latent_prepare", signature=sig)(
         dtype_code(rows.dtype), _ptr(rows), rows.stride(0), down_at, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(norm_weight), c_float(eps),
-        _ptr(slots), _ptr(c_pages), _ptr(kr_pages), T, heads, plain, rot, rank, 1 if interleaved else 0, _stream()), "latent_prepare")
+        _ptr(slots), _ptr(k_pages), _ptr(v_pages), _ptr(q_out), T, heads, plain, rot, rank, width, bs, 1 if interleaved else 0, _stream()),
+        "latent_prepare")
 
 
-def latent_attention(qa: torch.Tensor, rows: torch.Tensor, plain: int, rot: int, c_pages: torch.Tensor, kr_pages: torch.Tensor,
-                     block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, scale: float, window: int) -> torch.Tensor:
-    """softmax((qa . c_n + q_rot . kr_n) * scale) over the visible keys n (causal; the last ``window`` positions when
-    window > 0), times c_n: [T, heads, rank].  qa [T, heads, rank] contiguous; q_rot of head h at rows[:, h * (plain + rot) + plain:]."""
-    _on_gpu(qa, rows, c_pages, kr_pages, block_tables, cu_seqlens_q, seq_lens_k)
-    _need(qa.dim() == 3 and qa.is_contiguous() and rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[0] == qa.shape[0]
-          and rows.dtype == qa.dtype and c_pages.dtype == qa.dtype and kr_pages.dtype == qa.dtype, "latent_attention: operands of one type")
-    T, heads, rank = qa.shape
-    _need(rows.shape[1] >= heads * (plain + rot), "rows too narrow for the heads' rotated parts")
-    _need(rank <= MAX_LATENT_RANK and rot <= MAX_LATENT_ROT, f"latent sizes up to {MAX_LATENT_RANK} + {MAX_LATENT_ROT}")
-    _need(c_pages.dim() == 3 and c_pages.shape[2] == rank and kr_pages.shape == (*c_pages.shape[:2], rot) and c_pages.is_contiguous()
-          and kr_pages.is_contiguous(), "pages: [pages, block, rank] and [pages, block, rot]")
+def latent_attention(q: torch.Tensor, rank: int, rot: int, k_pages: torch.Tensor, block_tables: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                     seq_lens_k: torch.Tensor, scale: float, window: int) -> torch.Tensor:
+    """softmax(q . key_n * scale) over the visible keys n (causal; the last ``window`` positions when window > 0), times
+    c_n, the first ``rank`` elements of key row n: [T, heads, rank].  q [T, heads, width] contiguous rows [qa | q_rot | 0],
+    k_pages [pages, 1, block, width] rows [c | key part | 0].  For latents wider than the paged attention kernels take."""
+    _on_gpu(q, k_pages, block_tables, cu_seqlens_q, seq_lens_k)
+    _need(q.dim() == 3 and q.is_contiguous() and k_pages.dtype == q.dtype, "latent_attention: contiguous q [T, heads, width] of the pages' type")
+    T, heads, width = q.shape
+    _need(rank <= MAX_LATENT_RANK and rot <= MAX_LATENT_ROT and rank + rot <= width, f"latent sizes up to {MAX_LATENT_RANK} + {MAX_LATENT_ROT}")
+    _need(k_pages.dim() == 4 and k_pages.shape[1] == 1 and k_pages.shape[3] == width and k_pages.is_contiguous(), f"k_pages: [pages, 1, block, {width}]")
     S = seq_lens_k.numel()
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.stride(1) == 1,
           "block_tables: int32 [S, pages per sequence]")
     _need(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.numel() == S + 1 and seq_lens_k.dtype == torch.int32, "lengths: int32")
-    out = torch.empty((T, heads, rank), dtype=qa.dtype, device=qa.device)
-    sig = [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-           c_int, c_int, c_int, c_float, c_int, c_void_p]
+    out = torch.empty((T, heads, rank), dtype=q.dtype, device=q.device)
+    sig = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+           c_int, c_void_p]
     _check(_fn("latent_attention.hip", "pllm_latent_attention", signature=sig)(
-        dtype_code(qa.dtype), _ptr(qa), _ptr(rows), rows.stride(0), plain, _ptr(c_pages), _ptr(kr_pages), _ptr(out), _ptr(block_tables),
-        block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, heads, rank, rot, c_pages.shape[1], c_float(scale), window,
-        _stream()), "latent_attention")
+        dtype_code(q.dtype), _ptr(q), _ptr(k_pages), _ptr(out), _ptr(block_tables), block_tables.stride(0), _ptr(cu_seqlens_q),
+        _ptr(seq_lens_k), S, T, heads, rank, rot, width, k_pages.shape[2], c_float(scale), window, _stream()), "latent_attention")
     return out

@@ -1,0 +1,312 @@
+"""Gudutar in the engine against the plain implementation under tests/plain/: each mechanism alone, whole prompts,
+token-by-token decoding, portions down to two tokens, unequal requests in one batch with pages and state slots used
+again, the edges of the attention window and state carried over hundreds of tokens (with inputs made so that a fault
+shows), the first tokens of a sequence, sizes of several kinds, and greedy generation through ``LLMEngine``."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers
+from tests.gudutar_configs import ALONE, GUDU_A, GUDU_B
+from tests.helpers import TraceBuilder
+from tests.plain import gudutar_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {"A": GUDU_A, "B": GUDU_B, **ALONE}
+TOL = {"float32": 3e-5, "bfloat16": 6e-2}
+
+
+def write_folder(path, cfg, seed, stored, edit=None):
+    """A model folder with random weights (norm weights near one, everything else normal with the width's scale);
+    ``edit(tensors)`` may change them before they are stored."""
+    from safetensors.torch import load_file, save_file
+    from paged_llm_amd.weights import write_random_model
+    folder = write_random_model(str(path), cfg, seed=seed, dtype=stored, std=cfg["width"] ** -0.5, norm_jitter=True)
+    if edit is not None:
+        file = os.path.join(folder, "model.safetensors")
+        tensors = load_file(file)
+        edit(tensors)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, file)
+    return folder
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+
+    def get(name, stored):
+        if (name, stored) not in made:
+            made[name, stored] = write_folder(tmp_path_factory.mktemp(f"gudutar_{name}_{stored}"), CONFIGS[name],
+                                              seed=11 + len(name), stored=stored)
+        return made[name, stored]
+    return get
+
+
+_plain_cache: dict = {}
+
+
+def plain_logits(folder, tokens):
+    key = (folder, tuple(tokens))
+    if key not in _plain_cache:
+        _plain_cache[key] = plain.forward(plain.read_config(folder), plain.load_weights(folder), list(tokens)).numpy()
+    return _plain_cache[key]
+
+
+def session_for(folder, dtype, max_tokens, **kw):
+    from paged_llm_amd.engine.replay import ReplaySession
+    return ReplaySession(folder, dtype, max_tokens, None, **kw)
+
+
+def check(got: dict, folder, reqs: dict, dtype, tol=None):
+    tol = tol or TOL[dtype]
+    want = {rid: plain_logits(folder, toks) for rid, toks in reqs.items()}
+    errs = [helpers.worst(row, want[rid][pos]) for (rid, pos), row in got.items()]
+    worst_at = max(got, key=lambda k: helpers.worst(got[k], want[k[0]][k[1]]))
+    assert max(errs) <= tol, f"{worst_at}: {max(errs):.3g} (median {np.median(errs):.3g})"
+
+
+def rounded(n):
+    return -(-n // 64) * 64
+
+
+def whole(reqs):
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        trace.step([(rid, toks, "all")], end=[rid])
+    return trace
+
+
+def stored_as(dtype):
+    return "float32" if dtype == "float32" else "bfloat16"
+
+
+# --------------------------------------------------------------------------- each mechanism alone, and whole models
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_whole_prompts(folders, name, dtype):
+    folder = folders(name, stored_as(dtype))
+    vocab = CONFIGS[name]["vocab"]
+    reqs = {"p1": helpers.random_tokens(1, vocab, 1), "p5": helpers.random_tokens(5, vocab, 2), "p70": helpers.random_tokens(70, vocab, 3)}
+    got = helpers.replay_in_process(session_for(folder, dtype, 128), whole(reqs))
+    assert len(got) == 76
+    check(got, folder, reqs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "mamba2", "retention", "latent_attention"])
+def test_prompt_then_token_by_token(folders, name, dtype):
+    """A prompt in one step and then single tokens: cache, state slots and the window behind decoded tokens."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(75, CONFIGS[name]["vocab"], 7)
+    trace = TraceBuilder().step([("r", toks[:13], "all")])
+    for i in range(13, 75):
+        trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 74 else [])
+    session = session_for(folder, dtype, 128)
+    check(helpers.replay_in_process(session, trace), folder, {"r": toks}, dtype)
+    assert any(key[0] != "prompt" for key in session.runner._graphs), "single-token steps are replayed from graphs"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_token_by_token_from_the_first(folders, dtype):
+    """No prompt step at all: the first tokens meet the convolution's zeros and an empty state."""
+    folder = folders("A", stored_as(dtype))
+    toks = helpers.random_tokens(9, GUDU_A["vocab"], 8)
+    trace = TraceBuilder()
+    for i in range(9):
+        trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 8 else [])
+    check(helpers.replay_in_process(session_for(folder, dtype, 64), trace), folder, {"r": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("sizes", [[2], [3, 2, 7], [16, 1, 17, 2, 31], [64, 5]])
+def test_portions(folders, name, dtype, sizes):
+    """Prompts cut into portions of several sizes, down to two tokens (shorter than the convolution's reach), cut in the
+    middle of pages and of the window."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(97, CONFIGS[name]["vocab"], 9)
+    trace, at, k = TraceBuilder(), 0, 0
+    while at < len(toks):
+        n = min(sizes[k % len(sizes)], len(toks) - at)
+        trace.step([("r", toks[at:at + n], "all")], end=["r"] if at + n == len(toks) else [])
+        at, k = at + n, k + 1
+    check(helpers.replay_in_process(session_for(folder, dtype, 128), trace), folder, {"r": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_float32_logits_do_not_depend_on_the_cut(folders, name, dtype):
+    """The same request whole, in portions and token by token: equal within rounding of the compute type, and far
+    inside the bound against the plain implementation in float32."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(60, CONFIGS[name]["vocab"], 10)
+    a = helpers.replay_in_process(session_for(folder, dtype, 64), whole({"r": toks}))
+    trace = TraceBuilder().step([("r", toks[:31], "all")]).step([("r", toks[31:33], "all")])
+    for i in range(33, 60):
+        trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 59 else [])
+    b = helpers.replay_in_process(session_for(folder, dtype, 64), trace)
+    worst = max(helpers.worst(b[k], a[k]) for k in a)
+    assert worst <= (1e-5 if dtype == "float32" else 6e-2), worst
+
+
+# --------------------------------------------------------------------------- batches, pages and slots used again
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_batches_with_pages_and_slots_used_again(folders, name, dtype):
+    from tests.test_replay_gpu import mixed_trace
+    folder = folders(name, stored_as(dtype))
+    vocab = CONFIGS[name]["vocab"]
+    lengths = [33, 1, 90, 17, 64, 5, 48, 2, 71]
+    reqs = {f"q{i}": helpers.random_tokens(n, vocab, 40 + i) for i, n in enumerate(lengths)}
+    trace, peak = mixed_trace(reqs, max_live=3, seed=3)
+    session = session_for(folder, dtype, peak, max_requests=3)
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == sum(lengths)
+    check(got, folder, reqs, dtype)
+    session.manager.check_invariants()
+    assert session.manager.slots.num_free == session.manager.slots.num_slots == 3
+    assert all(session.manager.num_free_pages(g) == session.manager.num_pages(g) for g in session.manager.groups)
+    kinds = {"prompt" if key[0] == "prompt" else "decode" for key in session.runner._graphs}
+    assert kinds == {"prompt", "decode"}, "steps of both kinds were replayed from graphs"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_slot_that_held_another_request_starts_from_zero(folders, dtype):
+    """One state slot, one page pool of one request: the second request gets the slot and pages the first one left full."""
+    folder = folders("A", stored_as(dtype))
+    reqs = {"first": helpers.random_tokens(50, GUDU_A["vocab"], 60), "second": helpers.random_tokens(44, GUDU_A["vocab"], 61)}
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        trace.step([(rid, toks[:20], "all")])
+        trace.step([(rid, toks[20:22], "all")])
+        for i in range(22, len(toks)):
+            trace.step([(rid, toks[i:i + 1], "all")], end=[rid] if i == len(toks) - 1 else [])
+    session = session_for(folder, dtype, 64, max_requests=1)
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+
+
+# --------------------------------------------------------------------------- where random weights would hide a fault
+def _boost(token, factor):
+    def edit(tensors):
+        tensors["embed"][token] = (tensors["embed"][token].float() * factor).to(tensors["embed"].dtype)
+    return edit
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_edges_in_prompts_and_in_decoding(tmp_path, dtype):
+    """A token whose embedding is several times larger than the others' stands at one place; its key then dominates the
+    softmax of the queries that see it.  The positions at which it is last seen and first hidden (window - 1 and window
+    tokens later) are compared with the plain implementation, whole and decoded; the plain implementation with a window
+    one shorter or longer differs by far more than the bound there, so a window that is one token off would show."""
+    cfg = ALONE["latent_attention"]
+    window, special, at = cfg["layers"][0]["mixer"]["mask"]["size"], 7, 30
+    folder = write_folder(tmp_path, cfg, seed=5, stored=stored_as(dtype), edit=_boost(special, 6.0))
+    toks = [t if t != special else special + 1 for t in helpers.random_tokens(64, cfg["vocab"], 12)]
+    toks[at] = special
+    edge_in, edge_out = at + window - 1, at + window
+    want = plain_logits(folder, toks)
+    for off_by in (-1, 1):                                 # the plain implementation with another window: the test can tell
+        other = plain.read_config(folder)
+        other["layers"][0]["mixer"]["mask"]["size"] = window + off_by
+        moved = plain.forward(other, plain.load_weights(folder), toks).numpy()
+        pos = edge_in if off_by < 0 else edge_out
+        assert helpers.worst(moved[pos], want[pos]) > 10 * TOL[dtype], "the special token does not show at the window's edge"
+    for cut in (64, edge_in - 3, at + 1):                   # whole; the edge among decoded tokens; all of the window decoded
+        trace = TraceBuilder().step([("r", toks[:cut], "all")], end=["r"] if cut == 64 else [])
+        for i in range(cut, 64):
+            trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 63 else [])
+        got = helpers.replay_in_process(session_for(folder, dtype, 64), trace)
+        for pos in (edge_in - 1, edge_in, edge_out, edge_out + 1):
+            err = helpers.worst(got["r", pos], want[pos])
+            assert err <= TOL[dtype], f"cut {cut}, position {pos}: {err:.3g}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["retention", "mamba2"])
+def test_a_token_far_back_still_shows(tmp_path, name, dtype):
+    """The recurrent state carries one early, large token over hundreds of tokens, through portions, page borders and
+    decoded tokens; the plain implementation without that token differs far beyond the bound at the end, so a state
+    that was lost or reset on the way would show."""
+    cfg = ALONE[name]
+    if name == "retention":                                 # decays close to one, or nothing is left after 300 tokens
+        cfg = {**cfg, "layers": [{**cfg["layers"][0], "mixer": {**cfg["layers"][0]["mixer"], "decay": [0.999, 0.9999]}}]}
+    special = 3
+
+    def edit(tensors):
+        _boost(special, 8.0)(tensors)
+        if name == "mamba2":                                # slow decay: exp(A_log) small, so that the state keeps the token
+            tensors["l0.mix.A_log"] = torch.full_like(tensors["l0.mix.A_log"], -6.0)
+    folder = write_folder(tmp_path, cfg, seed=6, stored=stored_as(dtype), edit=edit)
+    toks = [t if t != special else special + 1 for t in helpers.random_tokens(330, cfg["vocab"], 13)]
+    toks[2] = special
+    want = plain_logits(folder, toks)
+    without = plain.forward(plain.read_config(folder), plain.load_weights(folder), toks[:2] + [special + 1] + toks[3:]).numpy()
+    assert helpers.worst(without[-1], want[-1]) > 10 * TOL[dtype], "the early token does not show at the end"
+    trace, at = TraceBuilder(), 0
+    for n in (17, 2, 64, 100, 3, 96):
+        trace.step([("r", toks[at:at + n], "last")])
+        at += n
+    for i in range(at, 330):
+        trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 329 else [])
+    check(helpers.replay_in_process(session_for(folder, dtype, 384), trace), folder, {"r": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    folder = folders("B", stored_as(dtype))
+    toks = helpers.random_tokens(300, GUDU_B["vocab"], 14)
+    trace = TraceBuilder().step([("r", toks[:4], "all")])
+    for i in range(4, 300):
+        trace.step([("r", toks[i:i + 1], "all" if i % 7 == 0 or i > 280 else [])], end=["r"] if i == 299 else [])
+    check(helpers.replay_in_process(session_for(folder, dtype, 320), trace), folder, {"r": toks}, dtype)
+
+
+# --------------------------------------------------------------------------- the entry point and its scheduler
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_engine(folders, name):
+    """``LLMEngine.generate`` with portions of 16 tokens, three requests at a time for five prompts (state slots and pages
+    are used again): in float32 the tokens are the plain implementation's greedy choice, in bfloat16 every row the engine
+    sampled from is within the bound of the plain logits along its own tokens."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    vocab = CONFIGS[name]["vocab"]
+    prompts = [helpers.random_tokens(n, vocab, 70 + n) for n in (3, 41, 18, 1, 29)]
+    for dtype in ("float32", "bfloat16"):
+        folder = folders(name, stored_as(dtype))
+        engine = LLMEngine(folder, EngineConfig(dtype=dtype, num_gpu_blocks=24, block_size=16, max_num_batched_tokens=16,
+                                                max_num_seqs=3, max_model_len=128))
+        rows = {}
+
+        def keep(requests, logits):
+            for r, row in zip(requests, logits.float().cpu()):
+                rows[r.id, len(r.tokens) - 1] = row.numpy()
+        engine.on_logits = keep
+        outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+        assert engine.cache_manager.slots.num_free == 3
+        for p, o in zip(prompts, outs):
+            assert len(o.token_ids) == 12
+            want = plain_logits(folder, p + o.token_ids)
+            for i, token in enumerate(o.token_ids):
+                pos = len(p) + i - 1
+                err = helpers.worst(rows[o.seq_id, pos], want[pos])
+                assert err <= TOL[dtype] and int(rows[o.seq_id, pos].argmax()) == token, (dtype, pos, err)
+                if dtype == "float32":
+                    top2 = np.sort(want[pos])[-2:]
+                    if top2[1] - top2[0] > 1e-3 * np.abs(want[pos]).max():
+                        assert token == int(want[pos].argmax()), (pos, token)
+
+
+def test_the_command_line_generates(folders, capsys):
+    import importlib.util
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("generate_example", os.path.join(root, "examples", "generate.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    code = mod.main(["--model", folders("A", "bfloat16"), "--prompt-ids", "5,6,7", "--prompt-ids", "9", "--max-tokens", "6",
+                     "--num-gpu-blocks", "16", "--max-model-len", "64", "--ignore-eos"])
+    out = capsys.readouterr().out
+    assert code == 0 and "decode_tokens=" in out and out.count("--- [") == 2

@@ -313,7 +313,7 @@ def test_toy_state_inside_replayed_graphs(toy_folder, dtype, tol):
     from paged_llm_amd.engine.replay import ReplaySession
     reqs = {f"g{i}": helpers.random_tokens(40 + i, TOY["vocab_size"], seed=260 + i) for i in range(5)}
     want = {rid: plain_toy(toy_folder, toks) for rid, toks in reqs.items()}
-    session = ReplaySession(toy_folder, dtype, 64 * 5, None)
+    session = ReplaySession(toy_folder, dtype, 64 * 5, None, max_requests=5)
     assert session.runner.use_graphs and session.runner.states
     trace = TraceBuilder()
     trace.step([(rid, toks[:9], "last") for rid, toks in reqs.items()])
