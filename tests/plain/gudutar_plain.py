@@ -35,6 +35,40 @@ def load_weights(model_dir: str) -> dict:
 
 
 # --------------------------------------------------------------------------- small pieces
+_NOISE = None      # a function applied to every product's operand rows and result (see ``rounding_noise``), or None
+
+
+def product(x, w):
+    """x W^T; with ``_NOISE`` set, rows and result are disturbed as a 16-bit compute type would round them."""
+    if _NOISE is None:
+        return x @ w.T
+    return _NOISE(_NOISE(x) @ w.T)
+
+
+class rounding_noise:
+    """Inside ``with rounding_noise(seed):`` every product's rows and result are multiplied by 1 + u * 2^-8 with u uniform
+    in (-1, 1), drawn from ``seed``: the relative error of two roundings to bfloat16, at random (an engine that computes
+    in bfloat16 rounds the rows, the result, and what it computes element by element between two products).  Several
+    seeds show how far the logits of one position move under the compute type's rounding alone; the state, the norms and
+    everything else that the design keeps in 32 bits stay exact."""
+
+    def __init__(self, seed: int, amplitude: float = 2.0 ** -8):
+        self.gen = torch.Generator().manual_seed(seed)
+        self.amplitude = amplitude
+
+    def __call__(self, t):
+        return t * (1.0 + (torch.rand(t.shape, generator=self.gen, dtype=t.dtype) * 2.0 - 1.0) * self.amplitude)
+
+    def __enter__(self):
+        global _NOISE
+        _NOISE = self
+        return self
+
+    def __exit__(self, *exc):
+        global _NOISE
+        _NOISE = None
+
+
 def gelu_tanh(z):
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
@@ -88,7 +122,7 @@ def mamba2_mixer(h, w: dict, m: dict, eps: float):
     L = h.shape[0]
     H, P, N, G, taps = m["heads"], m["vdim"], m["state"], m["groups"], m["conv"]
     inner = H * P
-    proj = h @ w["in"].T
+    proj = product(h, w["in"])
     z, xbc, dt = proj[:, :inner], proj[:, inner:2 * inner + 2 * G * N], proj[:, 2 * inner + 2 * G * N:]
     # causal convolution per channel: the last column of the filter meets the current token
     padded = torch.cat([torch.zeros(taps - 1, xbc.shape[1], dtype=h.dtype), xbc], dim=0)
@@ -112,16 +146,16 @@ def mamba2_mixer(h, w: dict, m: dict, eps: float):
     y = y.reshape(L, inner) * silu(z)
     parts = m["norm_groups"]
     y = unit_rms(y.reshape(L, parts, inner // parts), eps).reshape(L, inner) * w["norm"]
-    return y @ w["o"].T
+    return product(y, w["o"])
 
 
 def retention_mixer(h, w: dict, m: dict, eps: float):
     L = h.shape[0]
     H, d, P = m["heads"], m["dim"], m["vdim"]
     pos = torch.arange(L)
-    q = (h @ w["q"].T).reshape(L, H, d)
-    k = (h @ w["k"].T).reshape(L, H, d)
-    v = (h @ w["v"].T).reshape(L, H, P)
+    q = product(h, w["q"]).reshape(L, H, d)
+    k = product(h, w["k"]).reshape(L, H, d)
+    v = product(h, w["v"]).reshape(L, H, P)
     q = rotate(q, pos, m["rot"]["base"], m["rot"]["dims"], interleaved=False)
     k = rotate(k, pos, m["rot"]["base"], m["rot"]["dims"], interleaved=False) * d ** -0.5
     S = torch.zeros(H, d, P, dtype=h.dtype)
@@ -131,35 +165,37 @@ def retention_mixer(h, w: dict, m: dict, eps: float):
             S[a] = float(m["decay"][a]) * S[a] + torch.outer(k[t, a], v[t, a])
             o[t, a] = S[a].T @ q[t, a]
     o = unit_rms(o, eps).reshape(L, H * P)
-    return (o * silu(h @ w["g"].T)) @ w["o"].T
+    return product(o * silu(product(h, w["g"])), w["o"])
 
 
 def latent_attention_mixer(h, w: dict, m: dict, eps: float):
     L = h.shape[0]
     H, d, r, P, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     pos = torch.arange(L)
-    q = (h @ w["q"].T).reshape(L, H, d + r)
+    q = product(h, w["q"]).reshape(L, H, d + r)
     q_plain, q_rot = q[..., :d], q[..., d:]
-    down = h @ w["dkv"].T
+    down = product(h, w["dkv"])
     c = unit_rms(down[:, :rank], eps) * w["dkv.norm"]
     k_rot = down[:, rank:]                                              # [L, r], one for all heads
     base, dims = m["rot"]["base"], m["rot"]["dims"]
     q_rot = rotate(q_rot, pos, base, dims, interleaved=True)
     k_rot = rotate(k_rot, pos, base, dims, interleaved=True)
-    k_plain = (c @ w["uk"].T).reshape(L, H, d)
-    v = (c @ w["uv"].T).reshape(L, H, P)
+    k_plain = product(c, w["uk"]).reshape(L, H, d)
+    v = product(c, w["uv"]).reshape(L, H, P)
     i_idx, j_idx = pos[:, None], pos[None, :]
-    hidden = (j_idx > i_idx) | (i_idx - j_idx >= m["mask"]["size"])
+    hidden = j_idx > i_idx
+    if m.get("mask"):                                                   # a sliding window: query i sees 0 <= i - j < size
+        hidden = hidden | (i_idx - j_idx >= m["mask"]["size"])
     out = torch.zeros(L, H, P, dtype=h.dtype)
     for a in range(H):
         s = (q_plain[:, a] @ k_plain[:, a].T + q_rot[:, a] @ k_rot.T) * m["scale"]
         s = s.masked_fill(hidden, float("-inf"))
         out[:, a] = torch.softmax(s, dim=-1) @ v[:, a]
-    return out.reshape(L, H * P) @ w["o"].T
+    return product(out.reshape(L, H * P), w["o"])
 
 
 def dense_ff(h, w: dict):
-    return (gelu_tanh(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T
+    return product(gelu_tanh(product(h, w["gate"])) * product(h, w["up"]), w["down"])
 
 
 MIXERS = {"mamba2": mamba2_mixer, "retention": retention_mixer, "latent_attention": latent_attention_mixer}
@@ -185,4 +221,4 @@ def forward(cfg: dict, weights: dict, tokens: list, dtype=torch.float32, layers_
         if layers_out is not None:
             layers_out.append(x.clone())
     x = layer_norm(x, W["final.norm"], W["final.norm.b"], eps)
-    return x @ W["head"].T
+    return product(x, W["head"])

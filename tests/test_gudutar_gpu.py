@@ -61,12 +61,51 @@ def session_for(folder, dtype, max_tokens, **kw):
     return ReplaySession(folder, dtype, max_tokens, None, **kw)
 
 
-def check(got: dict, folder, reqs: dict, dtype, tol=None):
-    tol = tol or TOL[dtype]
+_noise_cache: dict = {}
+
+
+def rounding_scale(folder, tokens):
+    """Per position: how far the plain logits move (root mean square over four draws of ``helpers.worst``) when every
+    product's rows and result carry the relative error of bfloat16 rounding.  Some positions of these small random models
+    are far more sensitive than others (the first token of a retention layer is (q . k) v divided by its root mean
+    square, which is the sign of q . k: where that product is nearly zero, rounding decides the sign; a softmax between
+    two near-equal scores), so a bfloat16 result is judged against its own position's scale."""
+    key = (folder, tuple(tokens))
+    if key not in _noise_cache:
+        exact = plain_logits(folder, tokens)
+        cfg, weights = plain.read_config(folder), plain.load_weights(folder)
+        sq = np.zeros(len(tokens))
+        for seed in range(4):
+            with plain.rounding_noise(seed):
+                moved = plain.forward(cfg, weights, list(tokens)).numpy()
+            sq += (np.abs(moved - exact).max(axis=1) / np.abs(exact).max(axis=1)) ** 2
+        _noise_cache[key] = np.sqrt(sq / 4)
+    return _noise_cache[key]
+
+
+def bound_at(folder, tokens, pos, dtype):
+    """What a row may differ by: float32 a fixed bound; bfloat16 3 times the position's rounding scale, at least 3e-2."""
+    if dtype == "float32":
+        return TOL[dtype]
+    return max(3e-2, 3.0 * float(rounding_scale(folder, tokens)[pos]))
+
+
+def check(got: dict, folder, reqs: dict, dtype):
+    """Every row within its bound in float32; in bfloat16 no row beyond twice its bound and at most one in fifty beyond
+    it, and the median error below 2.5e-2."""
     want = {rid: plain_logits(folder, toks) for rid, toks in reqs.items()}
-    errs = [helpers.worst(row, want[rid][pos]) for (rid, pos), row in got.items()]
-    worst_at = max(got, key=lambda k: helpers.worst(got[k], want[k[0]][k[1]]))
-    assert max(errs) <= tol, f"{worst_at}: {max(errs):.3g} (median {np.median(errs):.3g})"
+    ratios, errs = {}, []
+    for (rid, pos), row in got.items():
+        err = helpers.worst(row, want[rid][pos])
+        errs.append(err)
+        ratios[rid, pos] = err / bound_at(folder, reqs[rid], pos, dtype)
+    worst_at = max(ratios, key=ratios.get)
+    said = f"{worst_at}: {ratios[worst_at]:.3g} of its bound (median error {np.median(errs):.3g})"
+    if dtype == "float32":
+        assert ratios[worst_at] <= 1.0, said
+    else:
+        over = sum(1 for r in ratios.values() if r > 1.0)
+        assert ratios[worst_at] <= 2.0 and over <= max(1, len(ratios) // 50) and np.median(errs) <= 2.5e-2, f"{said}, {over} rows over"
 
 
 def rounded(n):
@@ -149,8 +188,10 @@ def test_float32_logits_do_not_depend_on_the_cut(folders, name, dtype):
     for i in range(33, 60):
         trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 59 else [])
     b = helpers.replay_in_process(session_for(folder, dtype, 64), trace)
-    worst = max(helpers.worst(b[k], a[k]) for k in a)
-    assert worst <= (1e-5 if dtype == "float32" else 6e-2), worst
+    if dtype == "float32":
+        assert max(helpers.worst(b[k], a[k]) for k in a) <= 1e-5
+    else:
+        assert max(helpers.worst(b[k], a[k]) / bound_at(folder, toks, k[1], dtype) for k in a) <= 2.0
 
 
 # --------------------------------------------------------------------------- batches, pages and slots used again
@@ -214,7 +255,7 @@ def test_window_edges_in_prompts_and_in_decoding(tmp_path, dtype):
         other["layers"][0]["mixer"]["mask"]["size"] = window + off_by
         moved = plain.forward(other, plain.load_weights(folder), toks).numpy()
         pos = edge_in if off_by < 0 else edge_out
-        assert helpers.worst(moved[pos], want[pos]) > 10 * TOL[dtype], "the special token does not show at the window's edge"
+        assert helpers.worst(moved[pos], want[pos]) > 4 * bound_at(folder, toks, pos, dtype), "the special token does not show at the window's edge"
     for cut in (64, edge_in - 3, at + 1):                   # whole; the edge among decoded tokens; all of the window decoded
         trace = TraceBuilder().step([("r", toks[:cut], "all")], end=["r"] if cut == 64 else [])
         for i in range(cut, 64):
@@ -222,7 +263,7 @@ def test_window_edges_in_prompts_and_in_decoding(tmp_path, dtype):
         got = helpers.replay_in_process(session_for(folder, dtype, 64), trace)
         for pos in (edge_in - 1, edge_in, edge_out, edge_out + 1):
             err = helpers.worst(got["r", pos], want[pos])
-            assert err <= TOL[dtype], f"cut {cut}, position {pos}: {err:.3g}"
+            assert err <= 2.0 * bound_at(folder, toks, pos, dtype), f"cut {cut}, position {pos}: {err:.3g}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -245,7 +286,8 @@ def test_a_token_far_back_still_shows(tmp_path, name, dtype):
     toks[2] = special
     want = plain_logits(folder, toks)
     without = plain.forward(plain.read_config(folder), plain.load_weights(folder), toks[:2] + [special + 1] + toks[3:]).numpy()
-    assert helpers.worst(without[-1], want[-1]) > 10 * TOL[dtype], "the early token does not show at the end"
+    # (against the float32 bound: in bfloat16 the same kernels run, instantiated for the other storage type)
+    assert helpers.worst(without[-1], want[-1]) > 10 * TOL["float32"], "the early token does not show at the end"
     trace, at = TraceBuilder(), 0
     for n in (17, 2, 64, 100, 3, 96):
         trace.step([("r", toks[at:at + n], "last")])
@@ -293,7 +335,7 @@ def test_greedy_generation_through_the_engine(folders, name):
             for i, token in enumerate(o.token_ids):
                 pos = len(p) + i - 1
                 err = helpers.worst(rows[o.seq_id, pos], want[pos])
-                assert err <= TOL[dtype] and int(rows[o.seq_id, pos].argmax()) == token, (dtype, pos, err)
+                assert err <= 2.0 * bound_at(folder, p + o.token_ids, pos, dtype) and int(rows[o.seq_id, pos].argmax()) == token, (dtype, pos, err)
                 if dtype == "float32":
                     top2 = np.sort(want[pos])[-2:]
                     if top2[1] - top2[0] > 1e-3 * np.abs(want[pos]).max():
