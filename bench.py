@@ -43,6 +43,85 @@ MODELS = {
         TINYLLAMA, num_hidden_layers=32, hidden_size=4096, num_key_value_heads=8, head_dim=128, intermediate_size=14336,
         vocab_size=128256, rope_theta=500000.0, rope_scaling=_LLAMA3(8.0), max_position_embeddings=131072)),
 }
+
+
+def gudutar_config(width: int, periods: int, vocab: int, window: int = 1024) -> dict:
+    """Gudutar at sizes that resemble a real model's layers: ``periods`` times [state-space, state-space, retention,
+    latent attention with a feed-forward].  State-space layers of twice the width in heads of 64 channels with 128 state
+    rows; retention keys as wide as the model and values twice as wide, in heads of 256 / 512; sixteen attention heads of
+    128 + 64 query elements over a latent of 192 + 64 (one key row of 256 elements per token), a window of ``window``
+    positions; the feed-forward 2.75 times the width, as TinyLlama's."""
+    ssm = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+    heads = width // 256
+    ret = {"heads": heads, "dim": 256, "vdim": 512, "rot": {"base": 10000.0, "dims": 256},
+           "decay": [1.0 - 2.0 ** (-5 - h) for h in range(heads)]}
+    att = {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "mask": {"size": window},
+           "rot": {"base": 10000.0, "dims": 64}, "scale": (128 + 64) ** -0.5}
+    period = [{"type": "mamba2", "mixer": ssm, "mlp": None}, {"type": "mamba2", "mixer": ssm, "mlp": None},
+              {"type": "retention", "mixer": ret, "mlp": None},
+              {"type": "latent_attention", "mixer": att, "mlp": {"kind": "dense", "ff": 11 * width // 4}}]
+    return {"architecture": "Gudutar", "vocab": vocab, "width": width, "embedding": {"scale": float(width) ** 0.5}, "norm": {"eps": 1e-5},
+            "layers": [dict(l) for _ in range(periods) for l in period], "max_positions": 4096, "torch_dtype": "bfloat16"}
+
+
+def run_gudutar(dtype: str, context: int, steps: int, warmup: int, widths=(1024, 2048)) -> dict:
+    """Prefill (one prompt of 2048 tokens in one step) and decode (8 and 64 requests at ``context``) of Gudutar beside
+    the Llama decoder at the same width, number of layers, feed-forward width and vocabulary (random weights).  The
+    Llama model has a feed-forward on every layer and Gudutar on every fourth, so the pairs differ in weight; what is
+    compared is tokens per second and, per mixer, what its kernels take (see the profiles)."""
+    import torch
+    out = {}
+    for width in widths:
+        periods = 3
+        models = {
+            "gudutar": gudutar_config(width, periods, 32000),
+            "llama": dict(TINYLLAMA, num_hidden_layers=4 * periods, hidden_size=width, num_attention_heads=width // 64,
+                          num_key_value_heads=max(1, width // 512), head_dim=64, intermediate_size=11 * width // 4, torch_dtype=dtype),
+        }
+        for name, cfg in models.items():
+            row = {}
+            with tempfile.TemporaryDirectory() as folder:
+                engine = make_engine(cfg, folder, dtype, 64, context)
+                for tokens in (512, PREFILL_TOKENS):
+                    t = time_prefill(engine, tokens, seed=100 + tokens, repeats=4)
+                    row[f"prefill_{tokens}_ms"] = round(t * 1e3, 3)
+                    row[f"prefill_{tokens}_tok_per_s"] = round(tokens / t, 1)
+                for batch in (1, 8, 64):
+                    sec, _ = time_decode(engine, batch, context, steps, warmup, seed=batch)
+                    row[f"decode_b{batch}_ms"] = round(sec * 1e3, 4)
+                    row[f"decode_b{batch}_tok_per_s"] = round(batch / sec, 1)
+                params = sum(t.numel() for t in _weights_of(engine.model))
+                row["weights_millions"] = round(params / 1e6, 1)
+                del engine
+                torch.cuda.empty_cache()
+            out[f"{name}_w{width}"] = row
+    return out
+
+
+def _weights_of(model):
+    """The matrices a decode step streams (what the parts hold after loading)."""
+    seen = {}
+    def walk(obj, depth=0):
+        import torch
+        if isinstance(obj, torch.Tensor):
+            if obj.dim() >= 2:
+                seen[obj.data_ptr()] = obj
+        elif hasattr(obj, "plain") and hasattr(obj, "tiled"):
+            walk(obj.plain, depth + 1)
+        elif isinstance(obj, dict):
+            for v in obj.values():
+                walk(v, depth + 1)
+        elif isinstance(obj, (list, tuple)):
+            for v in obj:
+                walk(v, depth + 1)
+        elif hasattr(obj, "__dict__") and depth < 4 and type(obj).__module__.startswith("paged_llm_amd"):
+            for k, v in vars(obj).items():
+                if k not in ("cos", "sin", "position", "env"):
+                    walk(v, depth + 1)
+    walk([model.embedding, model.blocks, model.head])
+    return list(seen.values())
+
+
 # Published peaks of the MI355X: HBM3E bandwidth and dense MFMA rates.
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -552,6 +631,8 @@ def main() -> int:
                     "256 generated tokens each (use with --model llama-3.1-8b)")
     ap.add_argument("--prompt-sweep", default=None, metavar="N,N,...", help="prefill of one prompt of each of these lengths")
     ap.add_argument("--context-sweep", default=None, metavar="N,N,...", help="decode at --batch requests (and prefill up to 8192) at each of these contexts")
+    ap.add_argument("--gudutar", action="store_true", help="prefill and decode of the Gudutar decoder (state-space, retention and "
+                    "latent-attention layers) at two widths beside the Llama decoder of the same width and depth, instead")
     ap.add_argument("--kernels", action="store_true", help="every kernel of a decode step and of a prompt step on its own, with its fraction")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -569,6 +650,11 @@ def main() -> int:
     nbytes = 2 if short == "bf16" else 4
     numbers = model_numbers(cfg, nbytes)
 
+    if args.gudutar:
+        print(json.dumps({"metric": "Gudutar beside the Llama decoder at equal width, depth and vocabulary (random weights): prefill and decode",
+                          "dtype": short, "context": args.context,
+                          "models": run_gudutar(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2))}))
+        return 0
     if args.workload == "ragged64":
         print(json.dumps({"metric": f"output tokens/s, 64 ragged requests at once, prompts 64-2048 tokens, 256 generated each ({model_name}, random weights)",
                           "dtype": short, "unit": "tokens/s", "result": run_ragged64(cfg, args.dtype, model_name)}))

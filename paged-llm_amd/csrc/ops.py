@@ -1216,15 +1216,29 @@ def step_sizes(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> tu
     return dt, decay
 
 
+RECURRENCE_CHUNKS_FROM = 128      # tokens of the longest sequence of a step from which its recurrences run in chunks
+
+
+def recurrence_chunk(max_q_len: int, num_tokens: int) -> int:
+    """Tokens per chunk for a step's recurrences (0: every sequence token by token in one workgroup per head).  Chunks
+    spread a long portion over the GPU at the price of a workspace of one state per chunk, so they grow with the step."""
+    if max_q_len < RECURRENCE_CHUNKS_FROM:
+        return 0
+    return 64 if num_tokens <= 4096 else (128 if num_tokens <= 16384 else 256)
+
+
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, state_offset: int,
                       state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int,
-                      vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None) -> torch.Tensor:
+                      vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None, max_q_len: int = 0) -> torch.Tensor:
     """Per head:  S_t = decay_t S_(t-1) + k_t (vscale_t v_t)^T,   y_t = S_t^T q_t + skip v_t,   S [N, P] float32 at
     ``state[slot, state_offset + head * N * P :]``; a sequence with seq_starts == 0 starts from S = 0.
 
     q, k [T, key_heads, N] (views of one element type and one row stride, unit inner stride, heads side by side; head h
     uses key head h // (heads / key_heads)), v [T, heads, P] likewise, decay float32 [T, heads] or [heads] (one number
-    per head for all tokens), vscale float32 [T, heads] or None, skip float32 [heads] or None.  Returns y float32 [T, heads * P]."""
+    per head for all tokens), vscale float32 [T, heads] or None, skip float32 [heads] or None.  Returns y float32 [T, heads * P].
+    ``max_q_len``: a bound on the tokens of one sequence in this step (0: unknown); from ``RECURRENCE_CHUNKS_FROM`` on the
+    sequences are cut into chunks that run side by side (a chunk's own contribution from a zero state, the states carried
+    from chunk to chunk, the outputs from each chunk's true starting state), which rounds differently than token by token."""
     _on_gpu(q, k, v, decay, state, state_slots, seq_starts, cu_seqlens, vscale, skip)
     _need(q.dim() == 3 and q.shape == k.shape and q.dtype == k.dtype and q.stride() == k.stride() and q.stride(2) == 1
           and q.stride(1) == q.shape[2], "recurrence q, k: [T, key_heads, N] views of one layout with the heads side by side")
@@ -1238,12 +1252,16 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     _check_sequences(state, state_slots, seq_starts, cu_seqlens, num_seqs)
     _need(0 <= state_offset and state_offset + H * N * P <= state.shape[1], "the recurrence's state does not fit the state slot")
     out = torch.empty((T, H * P), dtype=torch.float32, device=v.device)
+    chunk = recurrence_chunk(max_q_len, T)
+    max_chunks = T // chunk + num_seqs if chunk else 0
+    ws_state = torch.empty((max_chunks, H * N * P), dtype=torch.float32, device=v.device) if chunk else None
+    ws_decay = torch.empty((max_chunks, H), dtype=torch.float32, device=v.device) if chunk else None
     sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
-           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
+           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     _check(_fn("recurrent.hip", "pllm_linear_recurrence", signature=sig)(
         _ptr(q), _ptr(k), dtype_code(q.dtype), q.stride(0), _ptr(v), dtype_code(v.dtype), v.stride(0), _ptr(decay), H if decay.dim() == 2 else 0,
         _ptr(vscale), _ptr(skip), state.data_ptr() + 4 * state_offset, state.stride(0), _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens),
-        _ptr(out), num_seqs, H, KH, N, P, _stream()), "linear_recurrence")
+        _ptr(out), num_seqs, H, KH, N, P, chunk, max_chunks, _ptr(ws_state), _ptr(ws_decay), _stream()), "linear_recurrence")
     return out
 
 

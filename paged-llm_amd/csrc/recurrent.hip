@@ -12,8 +12,7 @@
 //
 // A batch is token-major without padding: sequence s owns rows cu_seqlens[s] .. cu_seqlens[s + 1] - 1, its state
 // sits in slot state_slots[s], and seq_starts[s] == 0 says that it starts now, from a zero state, whatever the slot
-// held.  Sequences may have no rows at all.  All arithmetic is float; T is the storage type of rows.  Every token's
-// state update is done in one fixed order, so a sequence gives the same bits however it was cut into steps.
+// held.  Sequences may have no rows at all.  All arithmetic is float; T is the storage type of rows.
 #include "common.h"
 
 using namespace pllm;
@@ -184,37 +183,79 @@ struct RecurrenceArgs {
   int heads, key_heads, N, P, pblocks;
 };
 
-// One workgroup per (sequence, head, block of 64 value channels); lane = value channel, so a token's update needs no
-// exchange between lanes.  Wave w holds rows w * NR .. w * NR + NR - 1 of S in registers; with several waves their
-// partial outputs are added through LDS in wave order.  A token's k and q are fetched by one lane each and read out
-// lane by lane.
-template <int NR, int MAX_THREADS>
-__global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(RecurrenceArgs a) {
+// One workgroup per (sequence or chunk, head, block of 64 value channels); lane = value channel, so a token's update
+// needs no exchange between lanes.  Wave w holds rows w * NR .. w * NR + NR - 1 of S in registers; with several waves
+// their partial outputs are added through LDS in wave order.  A token's k and q are fetched by one lane each and read
+// out lane by lane.
+//
+// Three forms (MODE):
+//   kWhole       a sequence's tokens of this step one after the other, from the slot's state to the slot's state: steps
+//                of single tokens and short portions;
+//   kChunkState  long portions, first pass: the tokens of one chunk from a zero state, no outputs; leaves the chunk's
+//                own contribution S_loc and the product of its decays in the workspace;
+//   kChunkOut    third pass: a chunk's tokens from the state the sequence had when the chunk began (which the second
+//                pass, recurrence_carry_kernel, has put where S_loc was), with outputs, no state written.
+// With chunks, a long prompt's tokens are spread over the whole GPU instead of one workgroup per head; the additions
+// into S associate differently than token by token, so results differ from the whole form by float rounding.
+enum { kWhole = 0, kChunkState = 1, kChunkOut = 2 };
+
+struct ChunkArgs {
+  float* ws_state;      // [chunks][heads][N][P]
+  float* ws_decay;      // [chunks][heads]
+  int chunk;            // tokens per chunk
+  int num_seqs;
+};
+
+// Chunk j of the batch: sequences in order, each with ceil(q_len / chunk) chunks.  False when j is past the last one.
+__device__ __forceinline__ bool find_chunk(const int* __restrict__ cu_seqlens, int num_seqs, int chunk, int j, int& seq, int& local) {
+  int base = 0;
+  for (int s = 0; s < num_seqs; ++s) {
+    const int c = (cu_seqlens[s + 1] - cu_seqlens[s] + chunk - 1) / chunk;
+    if (j < base + c) { seq = s; local = j - base; return true; }
+    base += c;
+  }
+  return false;
+}
+
+template <int NR, int MAX_THREADS, int MODE>
+__global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(RecurrenceArgs a, ChunkArgs ca) {
   __shared__ float part[2][MAX_THREADS / 64][64];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, waves = blockDim.x >> 6;
   const int head = blockIdx.x / a.pblocks, pb = blockIdx.x % a.pblocks;
   const int p = pb * 64 + lane;
   const bool p_ok = p < a.P;
-  const int seq = blockIdx.y;
+  int seq = blockIdx.y, local = 0;
+  if (MODE != kWhole && !find_chunk(a.cu_seqlens, ca.num_seqs, ca.chunk, blockIdx.y, seq, local)) return;
   const int q_begin = a.cu_seqlens[seq], q_len = a.cu_seqlens[seq + 1] - q_begin;
   if (q_len <= 0) return;
+  const int t_first = MODE == kWhole ? 0 : local * ca.chunk;
+  const int t_last = MODE == kWhole ? q_len : (t_first + ca.chunk < q_len ? t_first + ca.chunk : q_len);
   const int kh = head / (a.heads / a.key_heads);
   const int n0 = wv * NR;
   const bool carried = a.seq_starts[seq] > 0;
-  float* st = a.state + (size_t)a.state_slots[seq] * a.slot_stride + (size_t)head * a.N * a.P;
+  float* st = MODE == kWhole ? a.state + (size_t)a.state_slots[seq] * a.slot_stride + (size_t)head * a.N * a.P
+                             : ca.ws_state + ((size_t)blockIdx.y * a.heads + head) * a.N * a.P;
   float S[NR];
 #pragma unroll
-  for (int i = 0; i < NR; ++i) S[i] = (carried && p_ok && n0 + i < a.N) ? st[(size_t)(n0 + i) * a.P + p] : 0.f;
+  for (int i = 0; i < NR; ++i)
+    S[i] = (MODE != kChunkState && (MODE == kChunkOut || carried) && p_ok && n0 + i < a.N) ? st[(size_t)(n0 + i) * a.P + p] : 0.f;
   const float skip = a.skip ? a.skip[head] : 0.f;
   const bool mine = lane < NR && n0 + lane < a.N;
-  for (int t = 0; t < q_len; ++t) {
+  float decays = 1.f;
+  for (int t = t_first; t < t_last; ++t) {
     const size_t row = (size_t)(q_begin + t);
     const size_t qk_at = row * a.qk_stride + (size_t)kh * a.N + n0 + lane;
     const float k_l = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
-    const float q_l = mine ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
+    const float q_l = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
     const float dec = a.decay[row * a.decay_stride + head];
     const float x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
     const float xg = a.vscale ? x * a.vscale[row * a.heads + head] : x;
+    if (MODE == kChunkState) {
+      decays *= dec;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) S[i] = fmaf(row_lane(k_l, i), xg, dec * S[i]);
+      continue;
+    }
     float y[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
@@ -233,32 +274,75 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     }
     if (wv == 0 && p_ok) a.out[row * (size_t)(a.heads * a.P) + (size_t)head * a.P + p] = fmaf(skip, x, total);
   }
+  if (MODE == kChunkOut) return;
   if (p_ok) {
 #pragma unroll
     for (int i = 0; i < NR; ++i)
       if (n0 + i < a.N) st[(size_t)(n0 + i) * a.P + p] = S[i];
   }
+  if (MODE == kChunkState && threadIdx.x == 0 && pb == 0) ca.ws_decay[(size_t)blockIdx.y * a.heads + head] = decays;
 }
 
+// Second pass: per sequence and state element, chunk after chunk:  ws[c] <- the state before chunk c,
+// S <- decays[c] * S + S_loc[c];  the state after the last chunk goes to the slot.
+__global__ __launch_bounds__(256) void recurrence_carry_kernel(RecurrenceArgs a, ChunkArgs ca) {
+  const size_t per_head = (size_t)a.N * a.P, per_seq = per_head * a.heads;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int seq = blockIdx.y;
+  if (idx >= per_seq) return;
+  const int q_len = a.cu_seqlens[seq + 1] - a.cu_seqlens[seq];
+  if (q_len <= 0) return;
+  int base = 0;
+  for (int s = 0; s < seq; ++s) base += (a.cu_seqlens[s + 1] - a.cu_seqlens[s] + ca.chunk - 1) / ca.chunk;
+  const int chunks = (q_len + ca.chunk - 1) / ca.chunk;
+  const int head = (int)(idx / per_head);
+  float* slot = a.state + (size_t)a.state_slots[seq] * a.slot_stride + idx;
+  float S = a.seq_starts[seq] > 0 ? *slot : 0.f;
+  for (int c = 0; c < chunks; ++c) {
+    float* w = ca.ws_state + (size_t)(base + c) * per_seq + idx;
+    const float loc = *w;
+    *w = S;
+    S = fmaf(ca.ws_decay[(size_t)(base + c) * a.heads + head], S, loc);
+  }
+  *slot = S;
+}
+
+template <int MODE>
+static void launch_recurrence(const RecurrenceArgs& a, const ChunkArgs& ca, dim3 grid, int waves, int need, hipStream_t stream) {
+  dim3 block(64 * waves);
+  if (waves > 4) hipLaunchKernelGGL((linear_recurrence_kernel<64, 1024, MODE>), grid, block, 0, stream, a, ca);
+  else if (need <= 8) hipLaunchKernelGGL((linear_recurrence_kernel<8, 256, MODE>), grid, block, 0, stream, a, ca);
+  else if (need <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<16, 256, MODE>), grid, block, 0, stream, a, ca);
+  else if (need <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<32, 256, MODE>), grid, block, 0, stream, a, ca);
+  else hipLaunchKernelGGL((linear_recurrence_kernel<64, 256, MODE>), grid, block, 0, stream, a, ca);
+}
+
+// chunk == 0: every sequence token by token in one workgroup per (head, block of channels).  chunk > 0: the three passes
+// over chunks of that many tokens; ws_state holds max_chunks * heads * N * P floats and ws_decay max_chunks * heads, with
+// max_chunks >= sum over the sequences of ceil(q_len / chunk) (total tokens / chunk + num_seqs is enough).
 PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, int qk_stride, const void* v, int v_dtype,
                                     int v_stride, const float* decay, int decay_stride, const float* vscale, const float* skip,
                                     float* state, long slot_stride, const int* state_slots, const int* seq_starts,
                                     const int* cu_seqlens, float* out, int num_seqs, int heads, int key_heads, int N, int P,
-                                    hipStream_t stream) {
+                                    int chunk, int max_chunks, float* ws_state, float* ws_decay, hipStream_t stream) {
   if (num_seqs <= 0) return 0;
   if (heads <= 0 || key_heads <= 0 || heads % key_heads || N <= 0 || N > 1024 || P <= 0) return -2;
+  if (chunk < 0 || (chunk > 0 && (max_chunks <= 0 || max_chunks > 65535 || !ws_state || !ws_decay)) || num_seqs > 65535) return -2;
   RecurrenceArgs a;
   a.q = q; a.k = k; a.v = v; a.decay = decay; a.vscale = vscale; a.skip = skip; a.state = state;
   a.state_slots = state_slots; a.seq_starts = seq_starts; a.cu_seqlens = cu_seqlens; a.out = out;
   a.slot_stride = slot_stride; a.qk_dtype = qk_dtype; a.qk_stride = qk_stride; a.v_dtype = v_dtype; a.v_stride = v_stride;
   a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = P; a.pblocks = (P + 63) / 64;
+  ChunkArgs ca{ws_state, ws_decay, chunk, num_seqs};
   const int waves = (N + 63) / 64, need = (N + waves - 1) / waves;   // rows of S per wave
-  dim3 grid(heads * a.pblocks, num_seqs), block(64 * waves);
-  if (waves > 4) hipLaunchKernelGGL((linear_recurrence_kernel<64, 1024>), grid, block, 0, stream, a);
-  else if (need <= 8) hipLaunchKernelGGL((linear_recurrence_kernel<8, 256>), grid, block, 0, stream, a);
-  else if (need <= 16) hipLaunchKernelGGL((linear_recurrence_kernel<16, 256>), grid, block, 0, stream, a);
-  else if (need <= 32) hipLaunchKernelGGL((linear_recurrence_kernel<32, 256>), grid, block, 0, stream, a);
-  else hipLaunchKernelGGL((linear_recurrence_kernel<64, 256>), grid, block, 0, stream, a);
+  if (chunk == 0) {
+    launch_recurrence<kWhole>(a, ca, dim3(heads * a.pblocks, num_seqs), waves, need, stream);
+  } else {
+    launch_recurrence<kChunkState>(a, ca, dim3(heads * a.pblocks, max_chunks), waves, need, stream);
+    const size_t per_seq = (size_t)heads * N * P;
+    hipLaunchKernelGGL(recurrence_carry_kernel, dim3((unsigned)((per_seq + 255) / 256), num_seqs), dim3(256), 0, stream, a, ca);
+    launch_recurrence<kChunkOut>(a, ca, dim3(heads * a.pblocks, max_chunks), waves, need, stream);
+  }
   PLLM_RETURN_LAST_ERROR();
 }
 

@@ -90,7 +90,7 @@ class Mamba2Mixer(_StatefulMixer):
         x = conv[:, :inner].unflatten(1, (self.heads, self.P))
         B = conv[:, inner:inner + gn].unflatten(1, (self.groups, self.N))
         C = conv[:, inner + gn:].unflatten(1, (self.groups, self.N))
-        y = ops.linear_recurrence(C, B, x, decay, state, 0, *seqs, vscale=dt, skip=w["D"])
+        y = ops.linear_recurrence(C, B, x, decay, state, 0, *seqs, vscale=dt, skip=w["D"], max_q_len=ctx.max_q_len)
         u = ops.gated_group_norm(y, z, w["norm"], inner // self.norm_groups, True, self.eps)
         return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
 
@@ -136,7 +136,8 @@ class RetentionMixer(_StatefulMixer):
         k = ops.rotary_to_float(rows[:, H * N:2 * H * N], ctx.positions, *tables, H, N, rot, inter, N ** -0.5)
         v = rows[:, 2 * H * N:2 * H * N + H * P].unflatten(1, (H, P))
         gate = rows[:, 2 * H * N + H * P:]
-        y = ops.linear_recurrence(q, k, v, self.decay, state, 0, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs)
+        y = ops.linear_recurrence(q, k, v, self.decay, state, 0, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs,
+                                  max_q_len=ctx.max_q_len)
         u = ops.gated_group_norm(y, gate, None, P, False, self.eps)
         return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
 
