@@ -72,6 +72,67 @@ __global__ void layernorm_kernel(const TI* __restrict__ in, const int* __restric
   }
 }
 
+// The same with the row in registers, four elements per thread and load (hidden a multiple of 4 up to kRowRegs * 1024,
+// rows on 16-byte boundaries in float and 8-byte ones in bfloat16): every value is read once.
+constexpr int kRowRegs = 4;
+
+template <typename T> struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void layernorm_regs_kernel(const TI* __restrict__ in, const int* __restrict__ row_index,
+                                                             const float* __restrict__ w, const float* __restrict__ b, float eps,
+                                                             float* stream_rows, TO* __restrict__ rows, int hidden) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
+  const TI* v = in + src * hidden;
+  float x[kRowRegs][4], add[kRowRegs][4];
+  float acc = 0.f;
+#pragma unroll
+  for (int j = 0; j < kRowRegs; ++j) {
+    const int at = (j * 256 + threadIdx.x) * 4;
+    if (at < hidden) {
+      const Quad<TI> q = *reinterpret_cast<const Quad<TI>*>(v + at);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { x[j][e] = to_f32(q.v[e]); acc += x[j][e]; }
+      if (stream_rows) {                                   // asked for early: it arrives while the sums are made
+        const float4 sv = *reinterpret_cast<const float4*>(stream_rows + (size_t)r * hidden + at);
+        add[j][0] = sv.x; add[j][1] = sv.y; add[j][2] = sv.z; add[j][3] = sv.w;
+      }
+    }
+  }
+  const float mean = block_sum(acc, scratch) / (float)hidden;
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < kRowRegs; ++j) {
+    const int at = (j * 256 + threadIdx.x) * 4;
+    if (at < hidden) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { const float d = x[j][e] - mean; sq = fmaf(d, d, sq); }
+    }
+  }
+  const float var = block_sum(sq, scratch) / (float)hidden;
+  const float inv = 1.f / sqrtf(var + eps);
+#pragma unroll
+  for (int j = 0; j < kRowRegs; ++j) {
+    const int at = (j * 256 + threadIdx.x) * 4;
+    if (at < hidden) {
+      const float4 wv = *reinterpret_cast<const float4*>(w + at), bv = *reinterpret_cast<const float4*>(b + at);
+      const float ww[4] = {wv.x, wv.y, wv.z, wv.w}, bb[4] = {bv.x, bv.y, bv.z, bv.w};
+      float y[4];
+      Quad<TO> o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        y[e] = (x[j][e] - mean) * inv * ww[e] + bb[e];
+        if (stream_rows) y[e] += add[j][e];
+        o.v[e] = from_f32<TO>(y[e]);
+      }
+      if (stream_rows) *reinterpret_cast<float4*>(stream_rows + (size_t)r * hidden + at) = make_float4(y[0], y[1], y[2], y[3]);
+      if (rows) *reinterpret_cast<Quad<TO>*>(rows + (size_t)r * hidden + at) = o;
+    }
+  }
+}
+
 // in_dtype / out_dtype: PLLM_F32 or PLLM_BF16.
 PLLM_API int pllm_layernorm(int in_dtype, int out_dtype, const void* in, const int* row_index, const float* w, const float* b,
                             float eps, float* stream_rows, void* rows, int num_rows, int hidden, hipStream_t stream) {
@@ -79,8 +140,15 @@ PLLM_API int pllm_layernorm(int in_dtype, int out_dtype, const void* in, const i
   if (hidden <= 0) return -2;
   dim3 grid(num_rows), block(256);
   const size_t lds = (size_t)(hidden + 16) * sizeof(float);
+  const bool in_regs = hidden % 4 == 0 && hidden <= kRowRegs * 1024 && (uintptr_t)in % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+                       (uintptr_t)b % 16 == 0 && (uintptr_t)stream_rows % 16 == 0 && (uintptr_t)rows % 16 == 0;
 #define PLLM_LN(TI, TO)                                                                                                          \
   do {                                                                                                                          \
+    if (in_regs) {                                                                                                              \
+      hipLaunchKernelGGL((layernorm_regs_kernel<TI, TO>), grid, block, 0, stream, (const TI*)in, row_index, w, b, eps,          \
+                         stream_rows, (TO*)rows, hidden);                                                                       \
+      break;                                                                                                                    \
+    }                                                                                                                           \
     if (lds > 48 * 1024) {                                                                                                      \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(layernorm_kernel<TI, TO>),                               \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                \

@@ -1137,6 +1137,11 @@ def gemm_heads(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None
     if out is None:
         out = torch.empty((T, heads, N), dtype=a.dtype, device=a.device)
     _need(out.shape == (T, heads, N) and out.stride(2) == 1 and out.dtype == a.dtype, "bad output for gemm_heads")
+    if a.dtype == torch.bfloat16:
+        # bfloat16: the vendor's batched product (as the other bfloat16 products of more than a few rows), straight into
+        # the output's rows through views with the heads in front
+        torch.bmm(a.transpose(0, 1), w.transpose(1, 2), out=out.transpose(0, 1))
+        return out
     sig = [c_int, c_int, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p]
     _check(_fn("gemm_generic.hip", "pllm_gemm_nt_batched", signature=sig)(
         dtype_code(a.dtype), dtype_code(out.dtype), _ptr(a), a.stride(0), a.stride(1), _ptr(w), K, N * K, _ptr(out), out.stride(0), out.stride(1),
@@ -1182,23 +1187,27 @@ def causal_conv(rows: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | N
 
 
 def rotary_to_float(rows: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, heads: int, head_dim: int,
-                    rot_dims: int, interleaved: bool, scale: float = 1.0) -> torch.Tensor:
+                    rot_dims: int, interleaved: bool, scale: float = 1.0, second_at: int | None = None, scale2: float = 1.0) -> torch.Tensor:
     """float32 [T, heads, head_dim]: the heads of ``rows`` [T, >= heads * head_dim] (unit inner stride) with their first
-    ``rot_dims`` elements turned by the tables' angles at ``positions``, times ``scale``."""
+    ``rot_dims`` elements turned by the tables' angles at ``positions``, times ``scale``.  With ``second_at``: float32
+    [2, T, heads, head_dim], the second set of heads being the one that starts ``second_at`` columns further in the rows,
+    times ``scale2`` (queries and keys of one product's rows in one launch)."""
     _on_gpu(rows, positions, cos, sin)
-    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= heads * head_dim, "rotary_to_float rows: [T, >= heads * head_dim]")
+    sets = 1 if second_at is None else 2
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= (second_at or 0) + heads * head_dim, "rotary_to_float rows: [T, >= heads * head_dim]")
     T = rows.shape[0]
     _need(positions.dtype == torch.int32 and positions.numel() == T and positions.is_contiguous(), "positions: int32 [T]")
     _need(rot_dims % 2 == 0 and 0 <= rot_dims <= head_dim, f"rotated width {rot_dims} of a head of {head_dim}")
     for t in (cos, sin):
         _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot_dims // 2 and t.is_contiguous(),
               f"rotary tables: float32 [positions, {rot_dims // 2}]")
-    out = torch.empty((T, heads, head_dim), dtype=torch.float32, device=rows.device)
-    sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]
+    out = torch.empty((sets, T, heads, head_dim), dtype=torch.float32, device=rows.device)
+    sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_long,
+           c_float, c_void_p]
     _check(_fn("recurrent.hip", "pllm_rotary_to_float", signature=sig)(
         dtype_code(rows.dtype), _ptr(rows), rows.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out), T, heads, head_dim, rot_dims,
-        1 if interleaved else 0, c_float(scale), _stream()), "rotary_to_float")
-    return out
+        1 if interleaved else 0, c_float(scale), sets, second_at or 0, T * heads * head_dim, c_float(scale2), _stream()), "rotary_to_float")
+    return out if sets == 2 else out[0]
 
 
 def step_sizes(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> tuple:
@@ -1229,13 +1238,16 @@ def recurrence_chunk(max_q_len: int, num_tokens: int) -> int:
 
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, state_offset: int,
                       state_slots: torch.Tensor, seq_starts: torch.Tensor, cu_seqlens: torch.Tensor, num_seqs: int,
-                      vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None, max_q_len: int = 0) -> torch.Tensor:
+                      vscale: torch.Tensor | None = None, skip: torch.Tensor | None = None, max_q_len: int = 0,
+                      step_sizes: tuple | None = None) -> torch.Tensor:
     """Per head:  S_t = decay_t S_(t-1) + k_t (vscale_t v_t)^T,   y_t = S_t^T q_t + skip v_t,   S [N, P] float32 at
     ``state[slot, state_offset + head * N * P :]``; a sequence with seq_starts == 0 starts from S = 0.
 
     q, k [T, key_heads, N] (views of one element type and one row stride, unit inner stride, heads side by side; head h
     uses key head h // (heads / key_heads)), v [T, heads, P] likewise, decay float32 [T, heads] or [heads] (one number
     per head for all tokens), vscale float32 [T, heads] or None, skip float32 [heads] or None.  Returns y float32 [T, heads * P].
+    ``step_sizes`` = (raw [T, heads] view with unit inner stride, bias float32 [heads], a_log float32 [heads]) in place of
+    ``decay`` (None) and ``vscale``: the kernel makes vscale_t = softplus(raw_t + bias) and decay_t = exp(-exp(a_log) vscale_t) itself.
     ``max_q_len``: a bound on the tokens of one sequence in this step (0: unknown); from ``RECURRENCE_CHUNKS_FROM`` on the
     sequences are cut into chunks that run side by side (a chunk's own contribution from a zero state, the states carried
     from chunk to chunk, the outputs from each chunk's true starting state), which rounds differently than token by token."""
@@ -1246,7 +1258,16 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     T, KH, N = q.shape
     H, P = v.shape[1], v.shape[2]
     _need(H % KH == 0 and 1 <= N <= 1024, f"{H} heads over {KH} key heads, N = {N} (at most 1024)")
-    _need(decay.dtype == torch.float32 and decay.is_contiguous() and tuple(decay.shape) in ((T, H), (H,)), f"decay: float32 [{T}, {H}] or [{H}]")
+    raw = raw_bias = a_log = None
+    if step_sizes is not None:
+        raw, raw_bias, a_log = step_sizes
+        _on_gpu(raw, raw_bias, a_log)
+        _need(decay is None and vscale is None, "step sizes take the place of decay and vscale")
+        _need(raw.shape == (T, H) and raw.stride(1) == 1, f"raw step sizes: [{T}, {H}] with unit inner stride")
+        for t in (raw_bias, a_log):
+            _need(t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous(), f"step sizes: float32 [{H}] per-head constants")
+    else:
+        _need(decay.dtype == torch.float32 and decay.is_contiguous() and tuple(decay.shape) in ((T, H), (H,)), f"decay: float32 [{T}, {H}] or [{H}]")
     _need(vscale is None or (vscale.dtype == torch.float32 and vscale.shape == (T, H) and vscale.is_contiguous()), f"vscale: float32 [{T}, {H}]")
     _need(skip is None or (skip.dtype == torch.float32 and skip.shape == (H,) and skip.is_contiguous()), f"skip: float32 [{H}]")
     _check_sequences(state, state_slots, seq_starts, cu_seqlens, num_seqs)
@@ -1256,11 +1277,15 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: 
     max_chunks = T // chunk + num_seqs if chunk else 0
     ws_state = torch.empty((max_chunks, H * N * P), dtype=torch.float32, device=v.device) if chunk else None
     ws_decay = torch.empty((max_chunks, H), dtype=torch.float32, device=v.device) if chunk else None
-    sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
+    sig = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+           c_void_p, c_int, c_int, c_void_p, c_void_p,
+           c_void_p, c_long, c_void_p, c_void_p,
            c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     _check(_fn("recurrent.hip", "pllm_linear_recurrence", signature=sig)(
-        _ptr(q), _ptr(k), dtype_code(q.dtype), q.stride(0), _ptr(v), dtype_code(v.dtype), v.stride(0), _ptr(decay), H if decay.dim() == 2 else 0,
-        _ptr(vscale), _ptr(skip), state.data_ptr() + 4 * state_offset, state.stride(0), _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens),
+        _ptr(q), _ptr(k), dtype_code(q.dtype), q.stride(0), _ptr(v), dtype_code(v.dtype), v.stride(0), _ptr(decay),
+        H if decay is not None and decay.dim() == 2 else 0, _ptr(vscale), _ptr(skip),
+        _ptr(raw), dtype_code(raw.dtype) if raw is not None else 0, raw.stride(0) if raw is not None else 0, _ptr(raw_bias), _ptr(a_log),
+        state.data_ptr() + 4 * state_offset, state.stride(0), _ptr(state_slots), _ptr(seq_starts), _ptr(cu_seqlens),
         _ptr(out), num_seqs, H, KH, N, P, chunk, max_chunks, _ptr(ws_state), _ptr(ws_decay), _stream()), "linear_recurrence")
     return out
 

@@ -32,9 +32,9 @@ constexpr int kConvChunk = 64;     // tokens of one sequence that one workgroup 
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_kernel(
     const T* __restrict__ in, int in_stride, const float* __restrict__ w, const float* __restrict__ bias,
-    const float* __restrict__ state, size_t slot_stride, const int* __restrict__ state_slots,
+    float* state, size_t slot_stride, const int* __restrict__ state_slots,
     const int* __restrict__ seq_starts, const int* __restrict__ cu_seqlens, T* __restrict__ out, int out_stride,
-    int channels, int taps, int act) {
+    int channels, int taps, int act, int leave_state) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int seq = blockIdx.y;
   const int q_begin = cu_seqlens[seq], q_len = cu_seqlens[seq + 1] - q_begin;
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   if (c >= channels || t0 >= q_len) return;
   const int t1 = t0 + kConvChunk < q_len ? t0 + kConvChunk : q_len;
   const bool carried = seq_starts[seq] > 0;
-  const float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * (taps - 1);
+  float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * (taps - 1);
   float wj[kMaxTaps], win[kMaxTaps];
 #pragma unroll
   for (int j = 0; j < kMaxTaps; ++j) {
@@ -70,6 +70,13 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
       else if (j == taps - 2) win[j] = cur;
     }
     out[(size_t)(q_begin + t) * out_stride + c] = from_f32<T>(act ? silu_f32(acc) : acc);
+  }
+  // With one chunk per sequence this thread alone has read the channel's state, and what it holds now are the last
+  // taps - 1 inputs: it leaves them itself (with several chunks another kernel does, after all of them have read).
+  if (leave_state) {
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j < taps - 1) st[j] = win[j];
   }
 }
 
@@ -107,16 +114,17 @@ PLLM_API int pllm_causal_conv(int dtype, const void* in, int in_stride, const fl
   if (taps < 1 || taps > kMaxTaps) return -2;
   dim3 block(256), grid((channels + 255) / 256, num_seqs, (max_q_len + kConvChunk - 1) / kConvChunk);
   dim3 grid_state((channels + 255) / 256, num_seqs);
+  const int fused = grid.z == 1 && taps > 1;
   if (dtype == PLLM_F32) {
     hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, stream, (const float*)in, in_stride, w, bias, state,
-                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (float*)out, out_stride, channels, taps, act);
-    if (taps > 1)
+                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (float*)out, out_stride, channels, taps, act, fused);
+    if (taps > 1 && !fused)
       hipLaunchKernelGGL(conv_state_update_kernel<float>, grid_state, block, 0, stream, (const float*)in, in_stride, state,
                          (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
   } else {
     hipLaunchKernelGGL(causal_conv_kernel<bf16>, grid, block, 0, stream, (const bf16*)in, in_stride, w, bias, state,
-                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (bf16*)out, out_stride, channels, taps, act);
-    if (taps > 1)
+                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (bf16*)out, out_stride, channels, taps, act, fused);
+    if (taps > 1 && !fused)
       hipLaunchKernelGGL(conv_state_update_kernel<bf16>, grid_state, block, 0, stream, (const bf16*)in, in_stride, state,
                          (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
   }
@@ -127,11 +135,15 @@ PLLM_API int pllm_causal_conv(int dtype, const void* in, int in_stride, const fl
 // out[t, h, i] = float(rotated in[t, h, i]) * scale: the first rot_dims elements of each head turn by the angle of the
 // token's position (tables cos/sin [positions, rot_dims / 2]); partners are (i, i + rot_dims / 2) or, interleaved,
 // (2i, 2i + 1).  The result stays in float.
+// blockIdx.y == 1: a second set of heads `second_at` columns further in the rows, into out + second_out, times scale2
+// (the keys behind the queries).
 template <typename T>
 __global__ void rotary_to_float_kernel(const T* __restrict__ in, int in_stride, const int* __restrict__ positions,
                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t, float* __restrict__ out,
-                                       int heads, int head_dim, int rot_dims, int interleaved, float scale) {
+                                       int heads, int head_dim, int rot_dims, int interleaved, float scale, int second_at,
+                                       size_t second_out, float scale2) {
   const int tok = blockIdx.x;
+  if (blockIdx.y == 1) { in += second_at; out += second_out; scale = scale2; }
   const int half = rot_dims / 2;
   const T* row = in + (size_t)tok * in_stride;
   const size_t table = (size_t)positions[tok] * half;
@@ -155,16 +167,17 @@ __global__ void rotary_to_float_kernel(const T* __restrict__ in, int in_stride, 
 
 PLLM_API int pllm_rotary_to_float(int dtype, const void* in, int in_stride, const int* positions, const float* cos_t,
                                   const float* sin_t, float* out, int num_tokens, int heads, int head_dim, int rot_dims,
-                                  int interleaved, float scale, hipStream_t stream) {
+                                  int interleaved, float scale, int sets, int second_at, long second_out, float scale2,
+                                  hipStream_t stream) {
   if (num_tokens <= 0) return 0;
-  if (rot_dims < 0 || rot_dims > head_dim || rot_dims % 2) return -2;
-  dim3 grid(num_tokens), block(256);
+  if (rot_dims < 0 || rot_dims > head_dim || rot_dims % 2 || sets < 1 || sets > 2) return -2;
+  dim3 grid(num_tokens, sets), block(256);
   if (dtype == PLLM_F32)
     hipLaunchKernelGGL(rotary_to_float_kernel<float>, grid, block, 0, stream, (const float*)in, in_stride, positions, cos_t, sin_t,
-                       out, heads, head_dim, rot_dims, interleaved, scale);
+                       out, heads, head_dim, rot_dims, interleaved, scale, second_at, (size_t)second_out, scale2);
   else
     hipLaunchKernelGGL(rotary_to_float_kernel<bf16>, grid, block, 0, stream, (const bf16*)in, in_stride, positions, cos_t, sin_t,
-                       out, heads, head_dim, rot_dims, interleaved, scale);
+                       out, heads, head_dim, rot_dims, interleaved, scale, second_at, (size_t)second_out, scale2);
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -174,6 +187,10 @@ struct RecurrenceArgs {
   const void* v;                       // [T, heads, P], element type v_dtype, row stride v_stride
   const float* decay;                  // a_t per head: decay[t * decay_stride + h] (decay_stride 0: one number per head)
   const float* vscale;                 // g_t per head [T, heads], or null for 1
+  // or both from raw step sizes [T, heads] (element type raw_dtype, row stride raw_stride):
+  //   g_t = softplus(raw + raw_bias[h]) (no clamp),  a_t = exp(-exp(a_log[h]) * g_t)
+  const void* raw; const float* raw_bias; const float* a_log;
+  int raw_dtype, raw_stride;
   const float* skip;                   // [heads] or null
   float* state;                        // slot s, head h: state + s * slot_stride + h * N * P, as [N][P]
   const int* state_slots; const int* seq_starts; const int* cu_seqlens;
@@ -240,6 +257,7 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
   for (int i = 0; i < NR; ++i)
     S[i] = (MODE != kChunkState && (MODE == kChunkOut || carried) && p_ok && n0 + i < a.N) ? st[(size_t)(n0 + i) * a.P + p] : 0.f;
   const float skip = a.skip ? a.skip[head] : 0.f;
+  const float rate = a.raw ? expf(a.a_log[head]) : 0.f, raw_bias = a.raw ? a.raw_bias[head] : 0.f;
   const bool mine = lane < NR && n0 + lane < a.N;
   float decays = 1.f;
   for (int t = t_first; t < t_last; ++t) {
@@ -247,9 +265,17 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     const size_t qk_at = row * a.qk_stride + (size_t)kh * a.N + n0 + lane;
     const float k_l = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
     const float q_l = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
-    const float dec = a.decay[row * a.decay_stride + head];
     const float x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
-    const float xg = a.vscale ? x * a.vscale[row * a.heads + head] : x;
+    float dec, xg;
+    if (a.raw) {
+      const float z = load_as_f32(a.raw, a.raw_dtype, row * a.raw_stride + head) + raw_bias;
+      const float step = z > 20.f ? z : log1pf(expf(z));
+      dec = expf(-rate * step);
+      xg = x * step;
+    } else {
+      dec = a.decay[row * a.decay_stride + head];
+      xg = a.vscale ? x * a.vscale[row * a.heads + head] : x;
+    }
     if (MODE == kChunkState) {
       decays *= dec;
 #pragma unroll
@@ -322,16 +348,19 @@ static void launch_recurrence(const RecurrenceArgs& a, const ChunkArgs& ca, dim3
 // max_chunks >= sum over the sequences of ceil(q_len / chunk) (total tokens / chunk + num_seqs is enough).
 PLLM_API int pllm_linear_recurrence(const void* q, const void* k, int qk_dtype, int qk_stride, const void* v, int v_dtype,
                                     int v_stride, const float* decay, int decay_stride, const float* vscale, const float* skip,
+                                    const void* raw, int raw_dtype, int raw_stride, const float* raw_bias, const float* a_log,
                                     float* state, long slot_stride, const int* state_slots, const int* seq_starts,
                                     const int* cu_seqlens, float* out, int num_seqs, int heads, int key_heads, int N, int P,
                                     int chunk, int max_chunks, float* ws_state, float* ws_decay, hipStream_t stream) {
   if (num_seqs <= 0) return 0;
   if (heads <= 0 || key_heads <= 0 || heads % key_heads || N <= 0 || N > 1024 || P <= 0) return -2;
+  if ((raw && (!raw_bias || !a_log)) || (!raw && !decay)) return -2;
   if (chunk < 0 || (chunk > 0 && (max_chunks <= 0 || max_chunks > 65535 || !ws_state || !ws_decay)) || num_seqs > 65535) return -2;
   RecurrenceArgs a;
   a.q = q; a.k = k; a.v = v; a.decay = decay; a.vscale = vscale; a.skip = skip; a.state = state;
   a.state_slots = state_slots; a.seq_starts = seq_starts; a.cu_seqlens = cu_seqlens; a.out = out;
   a.slot_stride = slot_stride; a.qk_dtype = qk_dtype; a.qk_stride = qk_stride; a.v_dtype = v_dtype; a.v_stride = v_stride;
+  a.raw = raw; a.raw_dtype = raw_dtype; a.raw_stride = raw_stride; a.raw_bias = raw_bias; a.a_log = a_log;
   a.decay_stride = decay_stride; a.heads = heads; a.key_heads = key_heads; a.N = N; a.P = P; a.pblocks = (P + 63) / 64;
   ChunkArgs ca{ws_state, ws_decay, chunk, num_seqs};
   const int waves = (N + 63) / 64, need = (N + waves - 1) / waves;   // rows of S per wave
@@ -412,16 +441,96 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __re
   }
 }
 
+// The same for groups whose channels a wave (or, with fewer groups than waves, a few waves side by side) holds in
+// registers: every value is read once, four channels per lane and load.  Needs group % 4 == 0, rows that start on
+// 16-byte (float) and 8-byte (bfloat16) boundaries, and at most kGroupRegs * 256 channels per wave.
+constexpr int kGroupRegs = 8;
+
+template <typename T> struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_regs_kernel(const float* __restrict__ y, const T* __restrict__ gate,
+                                                                    int gate_stride, const float* __restrict__ w, T* __restrict__ out,
+                                                                    int inner, int group, int gate_first, float eps) {
+  __shared__ float scratch[4];
+  const int row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int groups = inner / group;
+  const int parts = groups >= 4 ? 1 : 4 / groups;          // waves side by side on one group (groups 1 or 2; 3 gives 1)
+  const int slice = group / parts;                         // channels of a group that one wave takes
+  const float* yr = y + (size_t)row * inner;
+  const T* gr = gate + (size_t)row * gate_stride;
+  T* orow = out + (size_t)row * inner;
+  for (int g = wave / parts; g < groups; g += 4 / parts) {
+    const int base = g * group + (wave % parts) * slice;
+    float u[kGroupRegs][4], s[kGroupRegs][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kGroupRegs; ++j) {
+      const int at = (j * 64 + lane) * 4;
+      if (at < slice) {
+        const float4 yv = *reinterpret_cast<const float4*>(yr + base + at);
+        const Quad<T> gv = *reinterpret_cast<const Quad<T>*>(gr + base + at);
+        const float yy[4] = {yv.x, yv.y, yv.z, yv.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[j][e] = silu_f32(to_f32(gv.v[e]));
+          u[j][e] = gate_first ? yy[e] * s[j][e] : yy[e];
+          ss = fmaf(u[j][e], u[j][e], ss);
+        }
+      }
+    }
+    ss = wave_sum(ss);
+    if (parts > 1) {                                       // (then every wave runs this loop exactly once)
+      scratch[wave] = ss;
+      __syncthreads();
+      ss = 0.f;
+      for (int k = 0; k < parts; ++k) ss += scratch[(wave / parts) * parts + k];
+    }
+    const float inv = 1.f / sqrtf(ss / (float)group + eps);
+#pragma unroll
+    for (int j = 0; j < kGroupRegs; ++j) {
+      const int at = (j * 64 + lane) * 4;
+      if (at < slice) {
+        Quad<T> o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float r = gate_first ? u[j][e] * inv : (u[j][e] * inv) * s[j][e];
+          if (w) r *= w[base + at + e];
+          o.v[e] = from_f32<T>(r);
+        }
+        *reinterpret_cast<Quad<T>*>(orow + base + at) = o;
+      }
+    }
+  }
+}
+
+template <typename T>
+static bool group_norm_in_registers(const float* y, const void* gate, int gate_stride, void* out, int inner, int group) {
+  const int groups = inner / group, parts = groups >= 4 ? 1 : 4 / groups;
+  return group % (4 * parts) == 0 && group / parts <= kGroupRegs * 256 && inner % 4 == 0 && gate_stride % 4 == 0 &&
+         (uintptr_t)y % 16 == 0 && (uintptr_t)gate % (4 * sizeof(T)) == 0 && (uintptr_t)out % (4 * sizeof(T)) == 0;
+}
+
 PLLM_API int pllm_gated_group_norm(int dtype, const float* y, const void* gate, int gate_stride, const float* w, void* out,
                                    int num_tokens, int inner, int group, int gate_first, float eps, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (group <= 0 || inner % group) return -2;
   dim3 grid(num_tokens), block(256);
-  if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, y, (const float*)gate, gate_stride, w, (float*)out,
-                       inner, group, gate_first, eps);
-  else
-    hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
-                       inner, group, gate_first, eps);
+  if (dtype == PLLM_F32) {
+    if (group_norm_in_registers<float>(y, gate, gate_stride, out, inner, group))
+      hipLaunchKernelGGL(gated_group_norm_regs_kernel<float>, grid, block, 0, stream, y, (const float*)gate, gate_stride, w, (float*)out,
+                         inner, group, gate_first, eps);
+    else
+      hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, y, (const float*)gate, gate_stride, w, (float*)out,
+                         inner, group, gate_first, eps);
+  } else {
+    if (group_norm_in_registers<bf16>(y, gate, gate_stride, out, inner, group))
+      hipLaunchKernelGGL(gated_group_norm_regs_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
+                         inner, group, gate_first, eps);
+    else
+      hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, 0, stream, y, (const bf16*)gate, gate_stride, w, (bf16*)out,
+                         inner, group, gate_first, eps);
+  }
   PLLM_RETURN_LAST_ERROR();
 }

@@ -86,11 +86,11 @@ class Mamba2Mixer(_StatefulMixer):
         z, xbc, dt_raw = proj[:, :inner], proj[:, inner:inner + self.channels], proj[:, inner + self.channels:]
         seqs = (ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs)
         conv = ops.causal_conv(xbc, w["conv"], w["conv.b"], state, self.conv_at, *seqs, ctx.max_q_len)
-        dt, decay = ops.step_sizes(dt_raw, w["dt_bias"], w["A_log"])
         x = conv[:, :inner].unflatten(1, (self.heads, self.P))
         B = conv[:, inner:inner + gn].unflatten(1, (self.groups, self.N))
         C = conv[:, inner + gn:].unflatten(1, (self.groups, self.N))
-        y = ops.linear_recurrence(C, B, x, decay, state, 0, *seqs, vscale=dt, skip=w["D"], max_q_len=ctx.max_q_len)
+        y = ops.linear_recurrence(C, B, x, None, state, 0, *seqs, skip=w["D"], max_q_len=ctx.max_q_len,
+                                  step_sizes=(dt_raw, w["dt_bias"], w["A_log"]))
         u = ops.gated_group_norm(y, z, w["norm"], inner // self.norm_groups, True, self.eps)
         return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
 
@@ -132,8 +132,7 @@ class RetentionMixer(_StatefulMixer):
         rot = (pe.rotary_dim or N) if pe is not None else 0
         tables = (pe.cos, pe.sin) if pe is not None else (ctx.positions.new_zeros((1, 0), dtype=torch.float32),) * 2
         inter = bool(pe.interleaved) if pe is not None else False
-        q = ops.rotary_to_float(rows[:, :H * N], ctx.positions, *tables, H, N, rot, inter, 1.0)
-        k = ops.rotary_to_float(rows[:, H * N:2 * H * N], ctx.positions, *tables, H, N, rot, inter, N ** -0.5)
+        q, k = ops.rotary_to_float(rows, ctx.positions, *tables, H, N, rot, inter, 1.0, second_at=H * N, scale2=N ** -0.5)
         v = rows[:, 2 * H * N:2 * H * N + H * P].unflatten(1, (H, P))
         gate = rows[:, 2 * H * N + H * P:]
         y = ops.linear_recurrence(q, k, v, self.decay, state, 0, ctx.state_slots, ctx.seq_starts, ctx.cu_seqlens_q, ctx.num_seqs,
