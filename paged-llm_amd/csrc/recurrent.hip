@@ -260,21 +260,39 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
   const float rate = a.raw ? expf(a.a_log[head]) : 0.f, raw_bias = a.raw ? a.raw_bias[head] : 0.f;
   const bool mine = lane < NR && n0 + lane < a.N;
   float decays = 1.f;
-  for (int t = t_first; t < t_last; ++t) {
+  // What a token needs from memory is asked for one token ahead, so that it travels while the token before is computed.
+  struct Fetched { float k, q, x, a, g; };
+  auto fetch = [&](int t) {
+    Fetched f;
     const size_t row = (size_t)(q_begin + t);
     const size_t qk_at = row * a.qk_stride + (size_t)kh * a.N + n0 + lane;
-    const float k_l = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
-    const float q_l = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
-    const float x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
+    f.k = mine ? load_as_f32(a.k, a.qk_dtype, qk_at) : 0.f;
+    f.q = (MODE != kChunkState && mine) ? load_as_f32(a.q, a.qk_dtype, qk_at) : 0.f;
+    f.x = p_ok ? load_as_f32(a.v, a.v_dtype, row * a.v_stride + (size_t)head * a.P + p) : 0.f;
+    if (a.raw) {
+      f.a = load_as_f32(a.raw, a.raw_dtype, row * a.raw_stride + head);
+      f.g = 0.f;
+    } else {
+      f.a = a.decay[row * a.decay_stride + head];
+      f.g = a.vscale ? a.vscale[row * a.heads + head] : 1.f;
+    }
+    return f;
+  };
+  Fetched next = fetch(t_first);
+  for (int t = t_first; t < t_last; ++t) {
+    const Fetched cur = next;
+    if (t + 1 < t_last) next = fetch(t + 1);
+    const size_t row = (size_t)(q_begin + t);
+    const float k_l = cur.k, q_l = cur.q, x = cur.x;
     float dec, xg;
     if (a.raw) {
-      const float z = load_as_f32(a.raw, a.raw_dtype, row * a.raw_stride + head) + raw_bias;
+      const float z = cur.a + raw_bias;
       const float step = z > 20.f ? z : log1pf(expf(z));
       dec = expf(-rate * step);
       xg = x * step;
     } else {
-      dec = a.decay[row * a.decay_stride + head];
-      xg = a.vscale ? x * a.vscale[row * a.heads + head] : x;
+      dec = cur.a;
+      xg = x * cur.g;
     }
     if (MODE == kChunkState) {
       decays *= dec;

@@ -89,8 +89,14 @@ class Mamba2Mixer(_StatefulMixer):
         x = conv[:, :inner].unflatten(1, (self.heads, self.P))
         B = conv[:, inner:inner + gn].unflatten(1, (self.groups, self.N))
         C = conv[:, inner + gn:].unflatten(1, (self.groups, self.N))
-        y = ops.linear_recurrence(C, B, x, None, state, 0, *seqs, skip=w["D"], max_q_len=ctx.max_q_len,
-                                  step_sizes=(dt_raw, w["dt_bias"], w["A_log"]))
+        if ctx.max_q_len >= ops.RECURRENCE_CHUNKS_FROM:
+            # long portions: step sizes and decays by a kernel of their own, all tokens side by side (inside the recurrence
+            # their exponentials would stand in every token's way, twice: once per pass over the chunks)
+            dt, decay = ops.step_sizes(dt_raw, w["dt_bias"], w["A_log"])
+            y = ops.linear_recurrence(C, B, x, decay, state, 0, *seqs, vscale=dt, skip=w["D"], max_q_len=ctx.max_q_len)
+        else:
+            y = ops.linear_recurrence(C, B, x, None, state, 0, *seqs, skip=w["D"], max_q_len=ctx.max_q_len,
+                                      step_sizes=(dt_raw, w["dt_bias"], w["A_log"]))
         u = ops.gated_group_norm(y, z, w["norm"], inner // self.norm_groups, True, self.eps)
         return linear(u, self.w_o, out_dtype=_out_dtype(ctx))
 
