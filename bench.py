@@ -90,7 +90,7 @@ def run_gudutar(dtype: str, context: int, steps: int, warmup: int, widths=(1024,
                     sec, _ = time_decode(engine, batch, context, steps, warmup, seed=batch)
                     row[f"decode_b{batch}_ms"] = round(sec * 1e3, 4)
                     row[f"decode_b{batch}_tok_per_s"] = round(batch / sec, 1)
-                params = sum(t.numel() for t in _weights_of(engine.model))
+                params = sum(_weights_of(engine.model))
                 row["weights_millions"] = round(params / 1e6, 1)
                 del engine
                 torch.cuda.empty_cache()
@@ -99,27 +99,14 @@ def run_gudutar(dtype: str, context: int, steps: int, warmup: int, widths=(1024,
 
 
 def _weights_of(model):
-    """The matrices a decode step streams (what the parts hold after loading)."""
-    seen = {}
-    def walk(obj, depth=0):
-        import torch
-        if isinstance(obj, torch.Tensor):
-            if obj.dim() >= 2:
-                seen[obj.data_ptr()] = obj
-        elif hasattr(obj, "plain") and hasattr(obj, "tiled"):
-            walk(obj.plain, depth + 1)
-        elif isinstance(obj, dict):
-            for v in obj.values():
-                walk(v, depth + 1)
-        elif isinstance(obj, (list, tuple)):
-            for v in obj:
-                walk(v, depth + 1)
-        elif hasattr(obj, "__dict__") and depth < 4 and type(obj).__module__.startswith("paged_llm_amd"):
-            for k, v in vars(obj).items():
-                if k not in ("cos", "sin", "position", "env"):
-                    walk(v, depth + 1)
-    walk([model.embedding, model.blocks, model.head])
-    return list(seen.values())
+    """Numbers of elements of the tensors the model declares (what a checkpoint of it holds)."""
+    out = []
+    for spec in model.weight_specs().values():
+        n = 1
+        for d in spec.shape:
+            n *= d
+        out.append(n)
+    return out
 
 
 # Published peaks of the MI355X: HBM3E bandwidth and dense MFMA rates.

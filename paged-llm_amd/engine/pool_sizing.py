@@ -36,6 +36,12 @@ def pages_that_fit(model, config) -> int:
     free_now, total = torch.cuda.mem_get_info(device)
     # free memory, less the share of the device that is to stay unused, less room for a step's activations
     room = free_now - int(total * (1.0 - config.gpu_memory_utilization)) - step_peak
+    # mixers with a state of fixed size per request: one slot per request that may run, and the spare one
+    for spec in model.state_specs().values():
+        elems = 1
+        for d in spec.shape:
+            elems *= d
+        room -= (config.max_num_seqs + 1) * elems * torch.empty((), dtype=spec.dtype).element_size()
     page_bytes = sum(g.bytes_per_page(bs, model.dtype) for g in model.cache_groups().values())
     pages = room // max(1, page_bytes)
     ceiling = config.max_num_seqs * -(-config.max_model_len // bs)
