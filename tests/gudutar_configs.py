@@ -58,6 +58,15 @@ GUDU_B = model(64, 131, [
     _layer("latent_attention", _latent(heads=3, dim=8, rot_dim=4, vdim=8, kv_rank=40, window=16, base=50.0, scale=0.35), ff=40),
 ], eps=1e-4, scale=0.7)
 
+# Sizes that fit no vector load and no tile: a width that is no multiple of 4, odd head sizes, three norm parts of ten
+# channels, twelve state rows, a latent of 22 + 4 elements (padded to 32 in the pages), eight taps, a window of five.
+GUDU_C = model(50, 77, [
+    _layer("retention", _retention(heads=3, dim=10, vdim=6, rot_dims=6, base=33.0, decay=(0.6, 0.9, 0.99)), ff=34),
+    _layer("mamba2", _mamba(heads=3, vdim=10, state=12, groups=1, conv=8, norm_groups=3)),
+    _layer("latent_attention", _latent(heads=3, dim=6, rot_dim=4, vdim=10, kv_rank=22, window=5, base=7.0, scale=0.3)),
+    _layer("mamba2", None, weights_of=1),
+], eps=1e-3, scale=1.5)
+
 # One mechanism alone, each in the smallest model that holds it.
 ALONE = {
     "mamba2": model(48, 90, [_layer("mamba2", _mamba(heads=3, vdim=16, state=24, groups=3, conv=4, norm_groups=1))], scale=2.0),

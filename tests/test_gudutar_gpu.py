@@ -10,13 +10,13 @@ import pytest
 import torch
 
 from tests import helpers
-from tests.gudutar_configs import ALONE, GUDU_A, GUDU_B
+from tests.gudutar_configs import ALONE, GUDU_A, GUDU_B, GUDU_C
 from tests.helpers import TraceBuilder
 from tests.plain import gudutar_plain as plain
 
 pytestmark = pytest.mark.gpu
 
-CONFIGS = {"A": GUDU_A, "B": GUDU_B, **ALONE}
+CONFIGS = {"A": GUDU_A, "B": GUDU_B, "C": GUDU_C, **ALONE}
 TOL = {"float32": 3e-5, "bfloat16": 6e-2}
 
 
@@ -99,10 +99,10 @@ def float32_scale(folder, tokens):
 
 def bound_at(folder, tokens, pos, dtype, floor32=None):
     """What a row may differ by: in float32 3e-5, or 5 times the plain implementation's own float32 error at that position
-    if that is more; in bfloat16 3 times the position's rounding scale, at least 3e-2."""
+    if that is more; in bfloat16 4 times the position's rounding scale, at least 3e-2."""
     if dtype == "float32":
         return max(floor32 or TOL[dtype], 5.0 * float(float32_scale(folder, tokens)[pos]))
-    return max(3e-2, 3.0 * float(rounding_scale(folder, tokens)[pos]))
+    return max(3e-2, 4.0 * float(rounding_scale(folder, tokens)[pos]))
 
 
 def check(got: dict, folder, reqs: dict, dtype, floor32=None):
@@ -151,7 +151,7 @@ def test_whole_prompts(folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "mamba2", "retention", "latent_attention"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "mamba2", "retention", "latent_attention"])
 def test_prompt_then_token_by_token(folders, name, dtype):
     """A prompt in one step and then single tokens: cache, state slots and the window behind decoded tokens."""
     folder = folders(name, stored_as(dtype))
@@ -176,7 +176,7 @@ def test_token_by_token_from_the_first(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("sizes", [[2], [3, 2, 7], [16, 1, 17, 2, 31], [64, 5]])
 def test_portions(folders, name, dtype, sizes):
     """Prompts cut into portions of several sizes, down to two tokens (shorter than the convolution's reach), cut in the
@@ -210,7 +210,7 @@ def test_float32_logits_do_not_depend_on_the_cut(folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_long_portions_run_in_chunks(folders, name, dtype):
     """Portions of 128 tokens and more take the recurrences' chunked form (a chunk's own state from zero, the states
     carried from chunk to chunk, outputs from each chunk's starting state): lengths at, just past and between the
@@ -239,7 +239,7 @@ def test_long_portions_run_in_chunks(folders, name, dtype):
 
 # --------------------------------------------------------------------------- batches, pages and slots used again
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_mixed_batches_with_pages_and_slots_used_again(folders, name, dtype):
     from tests.test_replay_gpu import mixed_trace
     folder = folders(name, stored_as(dtype))
