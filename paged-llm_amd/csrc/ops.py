@@ -1150,7 +1150,7 @@ def gemm_heads(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None
 
 
 # ------------------------------------------------------------------------------------------- state of fixed size per request
-MAX_CONV_TAPS = 8
+MAX_CONV_TAPS = 16
 
 
 def _check_sequences(state: torch.Tensor, state_slots, seq_starts, cu_seqlens, num_seqs: int) -> None:

@@ -23,13 +23,13 @@ __device__ __forceinline__ float load_as_f32(const void* p, int dtype, size_t i)
 __device__ __forceinline__ float silu_f32(float z) { return z / (1.f + expf(-z)); }
 
 // ---------------------------------------------------------------------------------------------
-constexpr int kMaxTaps = 8;
+constexpr int kMaxTaps = 16;      // most taps of a filter; filters of up to 8 taps take the smaller instance of the kernels
 constexpr int kConvChunk = 64;     // tokens of one sequence that one workgroup walks
 
 // out[t, c] = act(bias[c] + sum_j w[c, j] * in[t - (taps - 1) + j, c]); the last column of w meets the current token;
 // inputs before the sequence's first token of this step come from the state (or are zero for a sequence that starts).
 // state: [slots][channels][taps - 1] floats, oldest input first.
-template <typename T>
+template <typename T, int MAXT>
 __global__ __launch_bounds__(256) void causal_conv_kernel(
     const T* __restrict__ in, int in_stride, const float* __restrict__ w, const float* __restrict__ bias,
     float* state, size_t slot_stride, const int* __restrict__ state_slots,
@@ -43,9 +43,9 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   const int t1 = t0 + kConvChunk < q_len ? t0 + kConvChunk : q_len;
   const bool carried = seq_starts[seq] > 0;
   float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * (taps - 1);
-  float wj[kMaxTaps], win[kMaxTaps];
+  float wj[MAXT], win[MAXT];
 #pragma unroll
-  for (int j = 0; j < kMaxTaps; ++j) {
+  for (int j = 0; j < MAXT; ++j) {
     wj[j] = j < taps ? w[(size_t)c * taps + j] : 0.f;
     win[j] = 0.f;
     if (j < taps - 1) {
@@ -59,13 +59,13 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     const float cur = to_f32(in[(size_t)(q_begin + t) * in_stride + c]);
     float acc = b;
 #pragma unroll
-    for (int j = 0; j < kMaxTaps - 1; ++j)
+    for (int j = 0; j < MAXT - 1; ++j)
       if (j < taps - 1) acc = fmaf(wj[j], win[j], acc);
 #pragma unroll
-    for (int j = 0; j < kMaxTaps; ++j)
+    for (int j = 0; j < MAXT; ++j)
       if (j == taps - 1) acc = fmaf(wj[j], cur, acc);
 #pragma unroll
-    for (int j = 0; j < kMaxTaps - 1; ++j) {
+    for (int j = 0; j < MAXT - 1; ++j) {
       if (j < taps - 2) win[j] = win[j + 1];
       else if (j == taps - 2) win[j] = cur;
     }
@@ -75,13 +75,13 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   // taps - 1 inputs: it leaves them itself (with several chunks another kernel does, after all of them have read).
   if (leave_state) {
 #pragma unroll
-    for (int j = 0; j < kMaxTaps - 1; ++j)
+    for (int j = 0; j < MAXT - 1; ++j)
       if (j < taps - 1) st[j] = win[j];
   }
 }
 
 // state[k] <- the input at token q_len - (taps - 1) + k of this step, or what the state held for it.
-template <typename T>
+template <typename T, int MAXT>
 __global__ __launch_bounds__(256) void conv_state_update_kernel(
     const T* __restrict__ in, int in_stride, float* state, size_t slot_stride, const int* __restrict__ state_slots,
     const int* __restrict__ seq_starts, const int* __restrict__ cu_seqlens, int channels, int taps) {
@@ -91,9 +91,9 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
   const int q_begin = cu_seqlens[seq], q_len = cu_seqlens[seq + 1] - q_begin;
   const bool carried = seq_starts[seq] > 0;
   float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * (taps - 1);
-  float nv[kMaxTaps];
+  float nv[MAXT];
 #pragma unroll
-  for (int k = 0; k < kMaxTaps - 1; ++k) {
+  for (int k = 0; k < MAXT - 1; ++k) {
     nv[k] = 0.f;
     if (k < taps - 1) {
       const int rel = q_len - (taps - 1) + k;
@@ -102,8 +102,22 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
     }
   }
 #pragma unroll
-  for (int k = 0; k < kMaxTaps - 1; ++k)
+  for (int k = 0; k < MAXT - 1; ++k)
     if (k < taps - 1) st[k] = nv[k];
+}
+
+template <typename T, int MAXT>
+static void launch_causal_conv(const void* in, int in_stride, const float* w, const float* bias, float* state, long slot_stride,
+                               const int* state_slots, const int* seq_starts, const int* cu_seqlens, void* out, int out_stride,
+                               int channels, int taps, int act, int num_seqs, int max_q_len, hipStream_t stream) {
+  dim3 block(256), grid((channels + 255) / 256, num_seqs, (max_q_len + kConvChunk - 1) / kConvChunk);
+  dim3 grid_state((channels + 255) / 256, num_seqs);
+  const int fused = grid.z == 1 && taps > 1;
+  hipLaunchKernelGGL((causal_conv_kernel<T, MAXT>), grid, block, 0, stream, (const T*)in, in_stride, w, bias, state,
+                     (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (T*)out, out_stride, channels, taps, act, fused);
+  if (taps > 1 && !fused)
+    hipLaunchKernelGGL((conv_state_update_kernel<T, MAXT>), grid_state, block, 0, stream, (const T*)in, in_stride, state,
+                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
 }
 
 PLLM_API int pllm_causal_conv(int dtype, const void* in, int in_stride, const float* w, const float* bias, float* state,
@@ -112,22 +126,11 @@ PLLM_API int pllm_causal_conv(int dtype, const void* in, int in_stride, const fl
                               hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len <= 0 || channels <= 0) return 0;
   if (taps < 1 || taps > kMaxTaps) return -2;
-  dim3 block(256), grid((channels + 255) / 256, num_seqs, (max_q_len + kConvChunk - 1) / kConvChunk);
-  dim3 grid_state((channels + 255) / 256, num_seqs);
-  const int fused = grid.z == 1 && taps > 1;
-  if (dtype == PLLM_F32) {
-    hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, stream, (const float*)in, in_stride, w, bias, state,
-                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (float*)out, out_stride, channels, taps, act, fused);
-    if (taps > 1 && !fused)
-      hipLaunchKernelGGL(conv_state_update_kernel<float>, grid_state, block, 0, stream, (const float*)in, in_stride, state,
-                         (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
-  } else {
-    hipLaunchKernelGGL(causal_conv_kernel<bf16>, grid, block, 0, stream, (const bf16*)in, in_stride, w, bias, state,
-                       (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, (bf16*)out, out_stride, channels, taps, act, fused);
-    if (taps > 1 && !fused)
-      hipLaunchKernelGGL(conv_state_update_kernel<bf16>, grid_state, block, 0, stream, (const bf16*)in, in_stride, state,
-                         (size_t)slot_stride, state_slots, seq_starts, cu_seqlens, channels, taps);
-  }
+#define PLLM_CONV(T, MAXT) launch_causal_conv<T, MAXT>(in, in_stride, w, bias, state, slot_stride, state_slots, seq_starts, cu_seqlens, \
+                                                       out, out_stride, channels, taps, act, num_seqs, max_q_len, stream)
+  if (dtype == PLLM_F32) { if (taps <= 8) PLLM_CONV(float, 8); else PLLM_CONV(float, kMaxTaps); }
+  else { if (taps <= 8) PLLM_CONV(bf16, 8); else PLLM_CONV(bf16, kMaxTaps); }
+#undef PLLM_CONV
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -278,10 +281,14 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
     }
     return f;
   };
-  Fetched next = fetch(t_first);
-  for (int t = t_first; t < t_last; ++t) {
+  // The state pass walks its chunk from the last token to the first: the chunk's own contribution is the sum over its
+  // tokens of k_t (g_t v_t)^T times the decays of the tokens behind t, and that product is at hand when t is reached
+  // from behind: one multiply-add per state row and token, no decay of the rows.
+  Fetched next = fetch(MODE == kChunkState ? t_last - 1 : t_first);
+  for (int n = t_first; n < t_last; ++n) {
+    const int t = MODE == kChunkState ? t_last - 1 - (n - t_first) : n;
     const Fetched cur = next;
-    if (t + 1 < t_last) next = fetch(t + 1);
+    if (n + 1 < t_last) next = fetch(MODE == kChunkState ? t - 1 : t + 1);
     const size_t row = (size_t)(q_begin + t);
     const float k_l = cur.k, q_l = cur.q, x = cur.x;
     float dec, xg;
@@ -295,9 +302,10 @@ __global__ __launch_bounds__(MAX_THREADS) void linear_recurrence_kernel(Recurren
       xg = x * cur.g;
     }
     if (MODE == kChunkState) {
-      decays *= dec;
+      const float xw = xg * decays;                       // decays: of the tokens behind t in the chunk
 #pragma unroll
-      for (int i = 0; i < NR; ++i) S[i] = fmaf(row_lane(k_l, i), xg, dec * S[i]);
+      for (int i = 0; i < NR; ++i) S[i] = fmaf(row_lane(k_l, i), xw, S[i]);
+      decays *= dec;
       continue;
     }
     float y[4] = {0.f, 0.f, 0.f, 0.f};

@@ -71,6 +71,7 @@ GUDU_C = model(50, 77, [
 ALONE = {
     "mamba2": model(48, 90, [_layer("mamba2", _mamba(heads=3, vdim=16, state=24, groups=3, conv=4, norm_groups=1))], scale=2.0),
     "mamba2_one_tap": model(48, 90, [_layer("mamba2", _mamba(heads=2, vdim=8, state=8, groups=1, conv=1, norm_groups=4))], scale=2.0),
+    "mamba2_many_state_rows": model(48, 90, [_layer("mamba2", _mamba(heads=2, vdim=8, state=272, groups=2, conv=9, norm_groups=1))], scale=2.0),
     "retention": model(48, 90, [_layer("retention", _retention(heads=2, dim=16, vdim=24, rot_dims=8, decay=(0.8, 0.99)))], scale=2.0),
     "latent_attention": model(48, 90, [_layer("latent_attention", _latent(heads=4, dim=16, rot_dim=16, vdim=12, kv_rank=32, window=9))], scale=2.0),
     "latent_attention_full": model(48, 90, [_layer("latent_attention", _latent(heads=1, dim=8, rot_dim=2, vdim=8, kv_rank=16, window=0))], scale=2.0),
