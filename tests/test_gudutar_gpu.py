@@ -105,7 +105,7 @@ def bound_at(folder, tokens, pos, dtype, floor32=None):
     return max(3e-2, 4.0 * float(rounding_scale(folder, tokens)[pos]))
 
 
-def check(got: dict, folder, reqs: dict, dtype, floor32=None):
+def check(got: dict, folder, reqs: dict, dtype, floor32=None, narrow=False):
     """Every row within its bound in float32 (``floor32``: another least bound than 3e-5); in bfloat16 no row beyond twice its bound and at most one in fifty beyond
     it, and the median error below 2.5e-2."""
     want = {rid: plain_logits(folder, toks) for rid, toks in reqs.items()}
@@ -120,7 +120,10 @@ def check(got: dict, folder, reqs: dict, dtype, floor32=None):
         assert ratios[worst_at] <= 1.0, said
     else:
         over = sum(1 for r in ratios.values() if r > 1.0)
-        assert ratios[worst_at] <= 2.0 and over <= max(1, len(ratios) // 50) and np.median(errs) <= 2.5e-2, f"{said}, {over} rows over"
+        # (narrow: models a few dozen channels wide, whose rows move more under rounding and whose few draws of the
+        #  yardstick say less: twice the allowances; a fault in a kernel moves most rows by their whole size)
+        most, middle = (4.0, 5e-2) if narrow else (2.0, 2.5e-2)
+        assert ratios[worst_at] <= most and over <= max(1, len(ratios) // 50) and np.median(errs) <= middle, f"{said}, {over} rows over"
 
 
 def rounded(n):
@@ -395,3 +398,77 @@ def test_the_command_line_generates(folders, capsys):
                      "--num-gpu-blocks", "16", "--max-model-len", "64", "--ignore-eos"])
     out = capsys.readouterr().out
     assert code == 0 and "decode_tokens=" in out and out.count("--- [") == 2
+
+
+# --------------------------------------------------------------------------- the replay program, and sizes drawn at random
+def test_the_replay_program(folders, tmp_path):
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = folders("A", "float32")
+    toks = {"a": helpers.random_tokens(70, GUDU_A["vocab"], 90), "b": helpers.random_tokens(45, GUDU_A["vocab"], 91)}
+    trace = TraceBuilder()
+    trace.step([("a", toks["a"][:50], [0, 49])])
+    trace.step([("a", toks["a"][50:52], "all"), ("b", toks["b"][:30], [])])
+    trace.step([("b", toks["b"][30:], "last"), ("a", toks["a"][52:53], "all")], end=["b"])
+    trace.step([("a", toks["a"][53:], "all")], end=["a"])
+    out_dir = tmp_path / "out"
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(out_dir),
+                           "--max-tokens", "192"], input=trace.jsonl(), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
+    got = helpers.read_replay_output(str(out_dir), trace, GUDU_A["vocab"])
+    assert len(got) == 2 + 2 + 1 + 1 + 17
+    check(got, folder, toks, "float32")
+
+
+def random_configuration(seed: int) -> dict:
+    """A Gudutar configuration with every size drawn at random (small ones, ones and odd ones included) and the three
+    mixers in a random order, some layers with borrowed weights."""
+    from tests.gudutar_configs import _latent, _layer, _mamba, _retention, model
+    rng = np.random.default_rng(seed)
+    pick = lambda *values: values[int(rng.integers(len(values)))]
+    made = {}
+
+    def mixer(kind):
+        if kind == "mamba2":
+            groups = pick(1, 2, 3)
+            heads = groups * pick(1, 2, 3)
+            vdim = pick(1, 2, 5, 8, 20, 33, 70)
+            parts = pick(*[d for d in (1, 2, 3, 4, 5) if (heads * vdim) % d == 0])
+            return _mamba(heads=heads, vdim=vdim, state=pick(1, 3, 16, 40, 64, 65, 130), groups=groups, conv=pick(1, 2, 4, 5), norm_groups=parts)
+        if kind == "retention":
+            heads, dim = pick(1, 2, 5), pick(2, 6, 16, 34, 70)
+            return _retention(heads=heads, dim=dim, vdim=pick(1, 3, 16, 40, 66), rot_dims=pick(*[d for d in (2, 4, 6, 16, 34) if d <= dim]),
+                              base=pick(10.0, 1e4, 1e6), decay=[float(rng.uniform(0.3, 0.9999)) for _ in range(heads)])
+        rot = pick(2, 4, 8, 18)
+        return _latent(heads=pick(1, 2, 5, 8), dim=pick(1, 4, 16, 30), rot_dim=rot, vdim=pick(1, 4, 24, 50), kv_rank=pick(3, 16, 40, 100, 260),
+                       window=pick(0, 1, 2, 7, 16, 33, 100), base=pick(10.0, 1e4), scale=float(rng.uniform(0.05, 0.5)))
+
+    layers = []
+    for i in range(int(rng.integers(2, 6))):
+        kind = pick("mamba2", "retention", "latent_attention")
+        if kind in made and rng.random() < 0.3:
+            layers.append(_layer(kind, None, weights_of=made[kind]))
+        else:
+            made.setdefault(kind, i)
+            layers.append(_layer(kind, mixer(kind), ff=pick(None, None, 10, 36, 65)))
+    return model(pick(16, 30, 48, 66, 100), pick(40, 97, 300), layers, eps=pick(1e-6, 1e-5, 1e-3), scale=float(rng.uniform(0.5, 12.0)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    """Whatever the sizes, the engine computes what the plain implementation computes, whole, in portions and token by
+    token, two requests side by side."""
+    cfg = random_configuration(seed)
+    folder = write_folder(tmp_path, cfg, seed=100 + seed, stored=stored_as(dtype))
+    reqs = {"a": helpers.random_tokens(150, cfg["vocab"], 200 + seed), "b": helpers.random_tokens(37, cfg["vocab"], 300 + seed)}
+    trace = TraceBuilder()
+    trace.step([("a", reqs["a"][:130], "all")])                                       # a long portion: the chunked recurrences
+    trace.step([("a", reqs["a"][130:132], "all"), ("b", reqs["b"][:20], "all")])
+    for i in range(17):
+        trace.step([("a", reqs["a"][132 + i:133 + i], "all"), ("b", reqs["b"][20 + i:21 + i], "all")], end=["b"] if i == 16 else [])
+    trace.step([("a", reqs["a"][149:], "all")], end=["a"])
+    got = helpers.replay_in_process(session_for(folder, dtype, 256), trace)
+    assert len(got) == 150 + 37
+    check(got, folder, reqs, dtype, floor32=3e-4, narrow=True)
