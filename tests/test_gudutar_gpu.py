@@ -472,3 +472,27 @@ def test_configurations_drawn_at_random(tmp_path, seed, dtype):
     got = helpers.replay_in_process(session_for(folder, dtype, 256), trace)
     assert len(got) == 150 + 37
     check(got, folder, reqs, dtype, floor32=3e-4, narrow=True)
+
+
+def test_preempted_requests_start_again_from_an_empty_state(folders):
+    """A page pool too small for three requests at once: the scheduler preempts the request admitted last (pages and state
+    slot given back, its tokens kept) and computes it again later as a longer prompt, from position 0 and so from a zero
+    state in whatever slot it gets.  Float32: the tokens are the plain implementation's greedy choice all the same."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    folder = folders("B", "float32")
+    vocab = GUDU_B["vocab"]
+    prompts = [helpers.random_tokens(n, vocab, 400 + n) for n in (30, 22, 27)]
+    engine = LLMEngine(folder, EngineConfig(dtype="float32", num_gpu_blocks=10, block_size=16, max_num_batched_tokens=32,
+                                            max_num_seqs=3, max_model_len=128))
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True))
+    assert engine.stats.num_preemptions > 0 and sum(o.num_preemptions for o in outs) > 0
+    assert engine.cache_manager.slots.num_free == 3
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 40
+        want = plain_logits(folder, p + o.token_ids)
+        for i, token in enumerate(o.token_ids):
+            row = want[len(p) + i - 1]
+            top2 = np.sort(row)[-2:]
+            if top2[1] - top2[0] > 1e-3 * np.abs(row).max():
+                assert token == int(row.argmax()), (len(p), i)
