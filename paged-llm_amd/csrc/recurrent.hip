@@ -55,8 +55,18 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     }
   }
   const float b = bias ? bias[c] : 0.f;
-  for (int t = t0; t < t1; ++t) {
-    const float cur = to_f32(in[(size_t)(q_begin + t) * in_stride + c]);
+  // Eight tokens' inputs are asked for at once: one wait for memory per eight tokens, not per token.
+  constexpr int kAhead = 8;
+  for (int tb = t0; tb < t1; tb += kAhead) {
+    T fetched[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u)
+      if (tb + u < t1) fetched[u] = in[(size_t)(q_begin + tb + u) * in_stride + c];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+    const int t = tb + u;
+    if (t >= t1) break;
+    const float cur = to_f32(fetched[u]);
     float acc = b;
 #pragma unroll
     for (int j = 0; j < MAXT - 1; ++j)
@@ -70,6 +80,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
       else if (j == taps - 2) win[j] = cur;
     }
     out[(size_t)(q_begin + t) * out_stride + c] = from_f32<T>(act ? silu_f32(acc) : acc);
+    }
   }
   // With one chunk per sequence this thread alone has read the channel's state, and what it holds now are the last
   // taps - 1 inputs: it leaves them itself (with several chunks another kernel does, after all of them have read).

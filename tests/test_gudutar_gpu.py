@@ -220,7 +220,7 @@ def test_long_portions_run_in_chunks(folders, name, dtype):
     chunks' borders, a second long portion that starts from a carried state, and short and single-token sequences beside
     a long one in the same step."""
     from paged_llm_amd.csrc import ops
-    assert ops.recurrence_chunk(128, 300) == 64 and ops.recurrence_chunk(127, 300) == 0
+    assert ops.recurrence_chunk(128, 300) == 16 and ops.recurrence_chunk(127, 300) == 0 and ops.recurrence_chunk(2048, 2048) == 64
     folder = folders(name, stored_as(dtype))
     vocab = CONFIGS[name]["vocab"]
     reqs = {"long": helpers.random_tokens(449, vocab, 20), "side": helpers.random_tokens(150, vocab, 21),
