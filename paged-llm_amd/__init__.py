@@ -1,4 +1,5 @@
-"""A paged Llama inference engine for one AMD MI355X (gfx950): model folder in, tokens out.
+"""A paged inference engine for one AMD MI355X (gfx950): model folder in, tokens out (the Llama decoder; Gudutar, a
+decoder of state-space, retention and latent-attention layers).
 
     from paged_llm_amd import EngineConfig, SamplingParams
     from paged_llm_amd.engine.llm_engine import LLMEngine
