@@ -26,17 +26,28 @@ from dataclasses import dataclass, field
 NO_PAGE = -1
 
 
+def first_visible_key(kind: str, window: int, position: int) -> int:
+    """The first position whose keys a query at ``position`` (and every later one) can still see in a group of that
+    kind: everything ("full"), the last ``window`` positions ("window"), or the block of ``window`` positions that the
+    query lies in, blocks counted from position 0 ("chunk")."""
+    if kind == "window":
+        return max(0, position - window + 1)
+    if kind == "chunk":
+        return (position // window) * window if position > 0 else 0
+    return 0
+
+
 @dataclass(frozen=True)
 class GroupSpec:
     name: str
-    kind: str = "full"        # "full" | "window"
-    window: int = 0           # positions kept, for kind "window"
+    kind: str = "full"        # "full" | "window" | "chunk"
+    window: int = 0           # positions kept, for kind "window"; positions of a block, for kind "chunk"
 
     def __post_init__(self):
-        if self.kind not in ("full", "window"):
+        if self.kind not in ("full", "window", "chunk"):
             raise ValueError(f"unknown cache group kind {self.kind!r}")
-        if self.kind == "window" and self.window <= 0:
-            raise ValueError("a windowed group needs window > 0")
+        if self.kind != "full" and self.window <= 0:
+            raise ValueError("a windowed or chunked group needs window > 0")
 
 
 @dataclass(frozen=True)
@@ -294,10 +305,7 @@ class CacheManager:
     # ------------------------------------------------------------------ allocation
     def _first_needed_page(self, g: GroupSpec, num_computed: int) -> int:
         """Pages below this index are out of the window of every query at position >= num_computed."""
-        if g.kind != "window":
-            return 0
-        first_key = num_computed - g.window + 1
-        return max(0, first_key) // self.block_size
+        return first_visible_key(g.kind, g.window, num_computed) // self.block_size
 
     def _nothing_to_do(self, hold: _Holding, num_computed: int, num_new: int, total_pages: int) -> bool:
         """The usual decode step: the pages are there, the one written to is the request's alone, and

@@ -8,7 +8,7 @@
 //   block_tables [num_seqs, bt_stride] int32; entry i holds positions i*block_size .. +block_size-1
 //   cu_seqlens_q [num_seqs+1], seq_lens_k [num_seqs] (context length including the new tokens)
 // Query i of a sequence sits at position seq_len_k - num_q + i and sees keys n <= that position
-// (and n > position - window when window > 0).  Query head j reads kv head j / (heads / kv_heads).
+// (and n > position - window when window > 0; with window < 0, only the keys of its own block of -window positions).  Query head j reads kv head j / (heads / kv_heads).
 // A score may carry further terms (a cap, a slope times the distance, a sink per head: ScoreTerms).
 //
 // Keys are walked in tiles of 64 aligned to absolute positions 0, 64, 128, ..., so the order of
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
   for (int i = lane; i < head_dim; i += 64) q_s[i] = to_f32(q[(size_t)tok * q_stride + (size_t)head * head_dim + i]);
   __syncthreads();
 
-  const int first_key = (window > 0 && q_pos - window + 1 > 0) ? q_pos - window + 1 : 0;
+  const int first_key = first_visible_key(q_pos, window);
   const int dims_per_lane = (head_dim + 63) / 64;  // <= 4
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   const int qpos_min = pos0 + col0 / G, qpos_max = pos0 + last_col / G;
   // Keys any column of this tile may see: [vis_lo, vis_hi)
   const int vis_hi = qpos_max + 1;
-  const int vis_lo = (window > 0 && qpos_min - window + 1 > 0) ? qpos_min - window + 1 : 0;
+  const int vis_lo = first_visible_key(qpos_min, window);
   int k_lo = vis_lo & ~63, k_hi = vis_hi;
   if (partition_size > 0) {
     k_lo = max(k_lo, part * partition_size);
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     my_valid[cb] = c < num_cols;
     const int tok = my_valid[cb] ? c / G : 0, hg = my_valid[cb] ? c - tok * G : 0;
     my_qpos[cb] = my_valid[cb] ? pos0 + tok : -1;               // -1: sees nothing
-    my_first[cb] = (window > 0 && my_qpos[cb] - window + 1 > 0) ? my_qpos[cb] - window + 1 : 0;
+    my_first[cb] = first_visible_key(my_qpos[cb], window);
     const size_t row = (size_t)(q_begin + tok) * q_stride + (size_t)(kvh * G + hg) * D;
     my_out[cb] = (size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D;
     if constexpr (kTerms) {
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   };
   auto compute_block = [&](KVBlock& blk, int n0) {
     // Every key of the block visible to every column?  Then no masking is needed.
-    const bool interior = (n0 + 63 <= qpos_min) && (n0 >= (window > 0 ? max(qpos_max - window + 1, 0) : 0)) && (n0 + 64 <= k_hi) &&
+    const bool interior = (n0 + 63 <= qpos_min) && (n0 >= first_visible_key(qpos_max, window)) && (n0 + 64 <= k_hi) &&
                           (col0 + 16 * NCB <= num_cols);
     // ---- S^T = K Q^T for four tiles of 16 keys
     floatx4 s_t[4][NCB];
@@ -577,7 +577,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
   const int wg_last = min(wg_col0 + kWgCols, num_cols) - 1;
   const int wg_qmin = pos0 + wg_col0 / G, wg_qmax = pos0 + wg_last / G;
   int k_hi = wg_qmax + 1;
-  int k_lo = ((window > 0 && wg_qmin - window + 1 > 0) ? wg_qmin - window + 1 : 0) & ~63;
+  int k_lo = first_visible_key(wg_qmin, window) & ~63;
   // With partitions (few tiles, long contexts: too few workgroups to fill the GPU otherwise) blockIdx.z takes one
   // aligned partition of the keys and leaves a partial result for the merge kernel.
   const int part = blockIdx.z;
@@ -592,7 +592,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
   const int last_col = min(col0 + 16 * NCB, num_cols) - 1;
   const int qpos_min = pos0 + col0 / G, qpos_max = wave_on ? pos0 + last_col / G : -1;
   const int vis_hi = qpos_max + 1;
-  const int vis_lo = (window > 0 && qpos_min - window + 1 > 0) ? qpos_min - window + 1 : 0;
+  const int vis_lo = first_visible_key(qpos_min, window);
 
   int my_qpos[NCB], my_first[NCB];
   bool my_valid[NCB];
@@ -605,7 +605,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
     my_valid[cb] = c < num_cols;
     const int tok = my_valid[cb] ? c / G : 0, hg = my_valid[cb] ? c - tok * G : 0;
     my_qpos[cb] = my_valid[cb] ? pos0 + tok : -1;
-    my_first[cb] = (window > 0 && my_qpos[cb] - window + 1 > 0) ? my_qpos[cb] - window + 1 : 0;
+    my_first[cb] = first_visible_key(my_qpos[cb], window);
     const size_t row = (size_t)(q_begin + tok) * q_stride + (size_t)(kvh * G + hg) * D;
     my_out[cb] = (size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D;
     if constexpr (kTerms) {
@@ -829,7 +829,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
       }
     }
   };
-  const int full_from = window > 0 ? max(qpos_max - window + 1, 0) : 0;   // blocks from here on are inside every column's window
+  const int full_from = first_visible_key(qpos_max, window);   // blocks from here on are inside every column's window
 
   // ---- the steps.  Step i is computed from LDS while the next steps are on their way in registers: two sets
   //      of them (steps i + 1 and i + 2) for head sizes up to 64, one set (step i + 1) where a second would not
@@ -982,7 +982,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     if (tok < q_begin || tok >= q_begin + num_q) return;           // a row of none of this launch's sequences
   }
   const int qpos = seq_lens_k[seq] - num_q + (tok - q_begin);
-  const int first_key = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  const int first_key = first_visible_key(qpos, window);
   const int p_lo = first_key / partition_size, p_hi = min(qpos / partition_size, num_partitions - 1);
   float M = (lane >= p_lo && lane <= p_hi) ? m_mine : -INFINITY;
   for (int p = 64 + lane; p <= p_hi; p += 64)

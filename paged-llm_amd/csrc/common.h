@@ -41,6 +41,15 @@ struct ScoreTerms {
   const float* sinks;   // [heads] floats or null
   __host__ __device__ bool any() const { return cap > 0.f || slopes || sinks; }
 };
+// The first key that a query at position `pos` sees under a causal mask given as one number: window > 0, the last
+// `window` positions (the query's own among them); window < 0, the keys of the query's own block of -window positions,
+// blocks counted from position 0 of the sequence; 0, every key.  It never decreases as `pos` grows.
+__device__ __forceinline__ int first_visible_key(int pos, int window) {
+  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (window < 0) return pos > 0 ? (pos / -window) * -window : 0;
+  return 0;
+}
+
 __device__ __forceinline__ float capped_score(float x, float cap) { return cap > 0.f ? cap * tanhf(x / cap) : x; }
 
 // One rotary pair turned by the angle whose cosine and sine are c and s.  Products and sums are rounded one by one (no

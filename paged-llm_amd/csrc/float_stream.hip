@@ -179,3 +179,93 @@ PLLM_API int pllm_round_rows(const float* x, void* rows, long n, hipStream_t str
   hipLaunchKernelGGL(round_rows_kernel, dim3(blocks), dim3(256), 0, stream, x, (bf16*)rows, (size_t)n);
   PLLM_RETURN_LAST_ERROR();
 }
+
+// ---------------------------------------------------------------------------------------------
+// RMS norms on both sides of a branch over a float stream, one row per workgroup:
+//   branch given:  y = branch[r] (+ bias);  stream[r] += mult * y / sqrt(mean(y^2) + eps) * w_branch      (in place)
+//   then, rows given:  rows[r] = T(s / sqrt(mean(s^2) + eps) * w_next)  with s the row of the stream as it is now
+//                      (w_next null: rows[r] = T(s), the stream in the compute type).
+// Without a branch the stream's row is src = row_index[r] (or r) and nothing is written to the stream.  The weights
+// are the factors themselves (an architecture that stores them around zero adds the one when it loads them).
+// `rows` has a row stride of its own, so that it may be a part of wider rows.
+template <typename TO>
+__global__ __launch_bounds__(256) void rms_sandwich_kernel(const float* __restrict__ branch, const float* __restrict__ bias,
+                                                           const float* __restrict__ w_branch, float mult, float* stream,
+                                                           const int* __restrict__ row_index, const float* __restrict__ w_next, float eps,
+                                                           TO* __restrict__ rows, long rows_stride, int hidden) {
+  extern __shared__ float lds[];
+  float* row = lds;               // [hidden]
+  float* scratch = lds + hidden;  // [16]
+  const int r = blockIdx.x;
+  const size_t src = (!branch && row_index) ? (size_t)row_index[r] : (size_t)r;
+  float* s = stream + src * hidden;
+  float sq = 0.f;
+  if (branch) {
+    const float* v = branch + (size_t)r * hidden;
+    float bsq = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float f = v[i] + (bias ? bias[i] : 0.f);
+      row[i] = f;
+      bsq = fmaf(f, f, bsq);
+    }
+    const float inv = 1.f / sqrtf(block_sum(bsq, scratch) / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float y = s[i] + mult * (row[i] * inv * w_branch[i]);
+      s[i] = y;
+      row[i] = y;
+      sq = fmaf(y, y, sq);
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float y = s[i];
+      row[i] = y;
+      sq = fmaf(y, y, sq);
+    }
+  }
+  if (!rows) return;
+  TO* out = rows + (size_t)r * rows_stride;
+  if (w_next) {
+    const float inv = 1.f / sqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = from_f32<TO>(row[i] * inv * w_next[i]);
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = from_f32<TO>(row[i]);
+  }
+}
+
+PLLM_API int pllm_rms_sandwich(int out_dtype, const float* branch, const float* bias, const float* w_branch, float mult, float* stream,
+                               const int* row_index, const float* w_next, float eps, void* rows, long rows_stride, int num_rows,
+                               int hidden, hipStream_t stream_) {
+  if (num_rows <= 0) return 0;
+  if (hidden <= 0 || !stream || (branch && !w_branch)) return -2;
+  const size_t lds = (size_t)(hidden + 16) * sizeof(float);
+  dim3 grid(num_rows), block(256);
+#define PLLM_SW(TO)                                                                                                        \
+  do {                                                                                                                    \
+    if (lds > 48 * 1024) {                                                                                                \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rms_sandwich_kernel<TO>),                          \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                          \
+      if (e != hipSuccess) return (int)e;                                                                                 \
+    }                                                                                                                     \
+    hipLaunchKernelGGL(rms_sandwich_kernel<TO>, grid, block, lds, stream_, branch, bias, w_branch, mult, stream, row_index, \
+                       w_next, eps, (TO*)rows, rows_stride, hidden);                                                      \
+  } while (0)
+  if (out_dtype == PLLM_F32) PLLM_SW(float); else PLLM_SW(bf16);
+#undef PLLM_SW
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, at : at + hidden] = T(x[t, :]): float rows into a part of wider rows of the compute type.
+template <typename TO>
+__global__ void place_rows_kernel(const float* __restrict__ x, TO* __restrict__ out, long out_stride, int hidden) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[(size_t)t * out_stride + i] = from_f32<TO>(x[(size_t)t * hidden + i]);
+}
+
+PLLM_API int pllm_place_rows(int out_dtype, const float* x, void* out, long out_stride, int num_rows, int hidden, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  dim3 grid(num_rows), block(256);
+  if (out_dtype == PLLM_F32) hipLaunchKernelGGL(place_rows_kernel<float>, grid, block, 0, stream, x, (float*)out, out_stride, hidden);
+  else hipLaunchKernelGGL(place_rows_kernel<bf16>, grid, block, 0, stream, x, (bf16*)out, out_stride, hidden);
+  PLLM_RETURN_LAST_ERROR();
+}

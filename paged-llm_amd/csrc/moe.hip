@@ -1,0 +1,244 @@
+// A feed-forward of routed experts: every token goes through `top` of `experts` small gated feed-forwards (and, where
+// the router says so, through pass-through experts that hand the token back), weighted by router scores.
+//
+//   moe_route      per token: router outputs in float, softmax over all of them, the choice among the best groups of
+//                  neighbouring experts by score + correction, the weights = the chosen experts' plain scores;
+//   moe_align      the (token, choice) pairs sorted by expert: per expert a run of rows, cut into tiles of rows;
+//   moe_expert_gemm the experts' products over those runs: act(gate h) * (up h) from the tokens' rows, and the down
+//                  product from the activations; one tile of rows per workgroup, every row's sums in ascending k,
+//                  so a pair's result does not depend on which other pairs share its tile or in which order;
+//   moe_combine    out[t] = sum over the token's choices, in their order, of weight * (expert output | the token's row).
+//
+// Router, softmax, weights and the final sum are float; T is the storage type of rows, activations and matrices.
+#include "common.h"
+
+using namespace pllm;
+
+constexpr int kMoeTileRows = 16;   // rows (pairs) of one tile of the experts' products
+
+// ---------------------------------------------------------------------------------------------
+// n = experts + pass-through experts router outputs; groups of n / groups neighbours; a group's mark is its largest
+// corrected score; only experts of the `keep` best groups can be chosen (ties: the lower index wins).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ router_w,
+                                                        const float* __restrict__ correction, int width, int n, int groups, int keep,
+                                                        int top, int* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ float lds[];
+  float* score = lds;            // [n]  router outputs, then scores
+  float* choice = lds + n;       // [n]  score + correction, -inf once taken or shut out
+  float* mark = lds + 2 * n;     // [groups]
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* row = h + (size_t)t * ld;
+  for (int e = wave; e < n; e += 4) {
+    const float* w = router_w + (size_t)e * width;
+    float acc = 0.f;
+    for (int i = lane; i < width; i += 64) acc = fmaf(to_f32(row[i]), w[i], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) score[e] = acc;
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  float m = -INFINITY;
+  for (int e = 0; e < n; ++e) m = fmaxf(m, score[e]);
+  float sum = 0.f;
+  for (int e = 0; e < n; ++e) { score[e] = expf(score[e] - m); sum += score[e]; }
+  const float inv = 1.f / sum;
+  for (int e = 0; e < n; ++e) {
+    score[e] *= inv;
+    choice[e] = score[e] + (correction ? correction[e] : 0.f);
+  }
+  const int per = n / groups;
+  if (keep < groups) {
+    for (int g = 0; g < groups; ++g) {
+      float best = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, choice[e]);
+      mark[g] = best;
+    }
+    // the `keep` best groups get +inf as their mark; the others' experts are shut out
+    for (int k = 0; k < keep; ++k) {
+      int at = -1;
+      float best = -INFINITY;
+      for (int g = 0; g < groups; ++g)
+        if (mark[g] != INFINITY && (at < 0 || mark[g] > best)) { at = g; best = mark[g]; }
+      mark[at] = INFINITY;
+    }
+    for (int g = 0; g < groups; ++g)
+      if (mark[g] != INFINITY)
+        for (int e = g * per; e < (g + 1) * per; ++e) choice[e] = -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) {
+    int at = 0;
+    float best = choice[0];
+    for (int e = 1; e < n; ++e)
+      if (choice[e] > best) { at = e; best = choice[e]; }
+    ids[(size_t)t * top + k] = at;
+    weights[(size_t)t * top + k] = score[at];
+    choice[at] = -INFINITY;
+  }
+}
+
+PLLM_API int pllm_moe_route(int dtype, const void* h, int ld, const float* router_w, const float* correction, int num_tokens, int width,
+                            int n, int groups, int keep, int top, int* ids, float* weights, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (n <= 0 || groups <= 0 || n % groups || keep <= 0 || keep > groups || top <= 0 || top > (n / groups) * keep) return -2;
+  const size_t lds = (size_t)(2 * n + groups) * sizeof(float);
+  if (lds > 48 * 1024) return -2;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, lds, stream, (const float*)h, ld, router_w, correction, width, n, groups, keep, top, ids, weights);
+  else
+    hipLaunchKernelGGL(moe_route_kernel<bf16>, grid, block, lds, stream, (const bf16*)h, ld, router_w, correction, width, n, groups, keep, top, ids, weights);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// ids [pairs] -> the pairs of experts < `experts` sorted by expert.
+//   sorted_pair [pairs]   the pair at each sorted row (rows past the last one: untouched)
+//   row_of_pair [pairs]   the sorted row of each pair, -1 for a pass-through expert
+//   tiles [max_tiles][3]  (expert, first row, rows) of every tile of at most kMoeTileRows rows; tiles[.][2] = 0 past the last
+// One workgroup; the order of the pairs of one expert is whatever the atomics give (the products do not depend on it).
+constexpr int kMoeMaxExperts = 1024;
+
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int pairs, int experts, int* __restrict__ sorted_pair,
+                                                         int* __restrict__ row_of_pair, int* __restrict__ tiles, int max_tiles) {
+  __shared__ int count[kMoeMaxExperts], first[kMoeMaxExperts], cursor[kMoeMaxExperts];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = at;
+      for (int r = 0; r < count[e] && nt < max_tiles; r += kMoeTileRows, ++nt) {
+        tiles[3 * nt] = e;
+        tiles[3 * nt + 1] = at + r;
+        tiles[3 * nt + 2] = min(kMoeTileRows, count[e] - r);
+      }
+      at += count[e];
+    }
+    for (; nt < max_tiles; ++nt) { tiles[3 * nt] = 0; tiles[3 * nt + 1] = 0; tiles[3 * nt + 2] = 0; }
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < experts) {
+      const int row = first[e] + atomicAdd(&cursor[e], 1);
+      sorted_pair[row] = p;
+      row_of_pair[p] = row;
+    } else {
+      row_of_pair[p] = -1;
+    }
+  }
+}
+
+PLLM_API int pllm_moe_align(const int* ids, int pairs, int experts, int* sorted_pair, int* row_of_pair, int* tiles, int max_tiles,
+                            hipStream_t stream) {
+  if (pairs <= 0) return 0;
+  if (experts <= 0 || experts > kMoeMaxExperts || max_tiles < (pairs + kMoeTileRows - 1) / kMoeTileRows + experts) return -2;
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, sorted_pair, row_of_pair, tiles, max_tiles);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// One tile of rows of one expert times 64 of the expert's weight rows, plain multiply-adds with float sums in ascending k.
+//   GATED: a[row] = rows_in[sorted_pair[row] / top] (the token's row), w = [gate; up] [experts, 2 n_out, K],
+//          out[row, n] = T(act(gate . a) * (up . a));
+//   else:  a[row] = rows_in[row] (the activations, already sorted), w [experts, n_out, K], out[row, n] = float sum.
+constexpr int kMoeCols = 64, kMoeK = 32;
+
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void moe_expert_gemm_kernel(const T* __restrict__ rows_in, int ld_in, const T* __restrict__ w,
+                                                              const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
+                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act) {
+  __shared__ float a_s[kMoeTileRows][kMoeK + 1];
+  __shared__ float w_s[(GATED ? 2 : 1) * kMoeCols][kMoeK + 1];
+  __shared__ int src[kMoeTileRows];
+  const int tile = blockIdx.x;
+  const int expert = tiles[3 * tile], row0 = tiles[3 * tile + 1], nrows = tiles[3 * tile + 2];
+  if (nrows <= 0) return;
+  const int n0 = blockIdx.y * kMoeCols;
+  const int tid = threadIdx.x;
+  if (tid < kMoeTileRows) src[tid] = tid < nrows ? (GATED ? sorted_pair[row0 + tid] / top : row0 + tid) : -1;
+  __syncthreads();
+  const T* we = w + (size_t)expert * (GATED ? 2 : 1) * n_out * K;
+  const int r = tid >> 4, cg = tid & 15;           // this thread: row r, columns cg, cg + 16, cg + 32, cg + 48
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc2[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += kMoeK) {
+    for (int i = tid; i < kMoeTileRows * kMoeK; i += 256) {
+      const int rr = i / kMoeK, kk = i - rr * kMoeK;
+      a_s[rr][kk] = (src[rr] >= 0 && k0 + kk < K) ? to_f32(rows_in[(size_t)src[rr] * ld_in + k0 + kk]) : 0.f;
+    }
+    for (int i = tid; i < (GATED ? 2 : 1) * kMoeCols * kMoeK; i += 256) {
+      const int cc = i / kMoeK, kk = i - cc * kMoeK;
+      const int half = cc / kMoeCols, col = n0 + (cc - half * kMoeCols);
+      w_s[cc][kk] = (col < n_out && k0 + kk < K) ? to_f32(we[((size_t)half * n_out + col) * K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < kMoeK; ++kk) {
+      const float a = a_s[r][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[j] = fmaf(a, w_s[cg + 16 * j][kk], acc[j]);
+        if (GATED) acc2[j] = fmaf(a, w_s[kMoeCols + cg + 16 * j][kk], acc2[j]);
+      }
+    }
+    __syncthreads();
+  }
+  if (r >= nrows) return;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int col = n0 + cg + 16 * j;
+    if (col >= n_out) continue;
+    if (GATED) reinterpret_cast<T*>(out_)[(size_t)(row0 + r) * ld_out + col] = from_f32<T>(gate_activation(acc[j], act) * acc2[j]);
+    else reinterpret_cast<float*>(out_)[(size_t)(row0 + r) * ld_out + col] = acc[j];
+  }
+}
+
+PLLM_API int pllm_moe_expert_gemm(int dtype, int gated, const void* rows_in, int ld_in, const void* w, const int* tiles, int max_tiles,
+                                  const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, hipStream_t stream) {
+  if (max_tiles <= 0) return 0;
+  if (n_out <= 0 || K <= 0 || top <= 0 || act < 0 || act >= PLLM_ACT_COUNT) return -2;
+  dim3 grid(max_tiles, (n_out + kMoeCols - 1) / kMoeCols), block(256);
+#define PLLM_MOE(T, G)                                                                                                         \
+  hipLaunchKernelGGL((moe_expert_gemm_kernel<T, G>), grid, block, 0, stream, (const T*)rows_in, ld_in, (const T*)w, tiles,    \
+                     sorted_pair, top, n_out, K, out, ld_out, act)
+  if (dtype == PLLM_F32) { if (gated) PLLM_MOE(float, true); else PLLM_MOE(float, false); }
+  else { if (gated) PLLM_MOE(bf16, true); else PLLM_MOE(bf16, false); }
+#undef PLLM_MOE
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, :] = sum_k weights[t, k] * (row_of_pair[t, k] >= 0 ? expert_out[row_of_pair[t, k], :] : h[t, :]), in the order of k.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ expert_out, const T* __restrict__ h, int ld_h,
+                                                          const int* __restrict__ row_of_pair, const float* __restrict__ weights,
+                                                          int top, int width, float* __restrict__ out) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int row = row_of_pair[(size_t)t * top + k];
+      const float v = row >= 0 ? expert_out[(size_t)row * width + i] : to_f32(h[(size_t)t * ld_h + i]);
+      acc = fmaf(weights[(size_t)t * top + k], v, acc);
+    }
+    out[(size_t)t * width + i] = acc;
+  }
+}
+
+PLLM_API int pllm_moe_combine(int dtype, const float* expert_out, const void* h, int ld_h, const int* row_of_pair, const float* weights,
+                              int num_tokens, int top, int width, float* out, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, expert_out, (const float*)h, ld_h, row_of_pair, weights, top, width, out);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, block, 0, stream, expert_out, (const bf16*)h, ld_h, row_of_pair, weights, top, width, out);
+  PLLM_RETURN_LAST_ERROR();
+}

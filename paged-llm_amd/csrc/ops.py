@@ -1372,3 +1372,196 @@ def latent_attention(q: torch.Tensor, rank: int, rot: int, k_pages: torch.Tensor
         dtype_code(q.dtype), _ptr(q), _ptr(k_pages), _ptr(out), _ptr(block_tables), block_tables.stride(0), _ptr(cu_seqlens_q),
         _ptr(seq_lens_k), S, T, heads, rank, rot, width, k_pages.shape[2], c_float(scale), window, _stream()), "latent_attention")
     return out
+
+
+# ------------------------------------------------------------------------------------------- norms on both sides of a branch
+def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: torch.Tensor | None, mult: float, eps: float,
+                 w_next: torch.Tensor | None = None, out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+                 bias: torch.Tensor | None = None, row_index: torch.Tensor | None = None) -> torch.Tensor | None:
+    """RMS norms around a float32 residual stream, all in float.  With ``branch`` (float32 rows like the stream):
+    stream += mult * rms_norm(branch + bias) * w_branch, in place.  Then, when ``out`` or ``out_dtype`` is given, the
+    rows of the stream as it is now are returned in that type: normed and times ``w_next``, or as they are when
+    ``w_next`` is None.  ``out`` may be a view with a row stride of its own (unit inner stride).  Without a branch
+    ``row_index`` (int32) picks the rows of the stream; nothing is written to the stream then."""
+    _on_gpu(stream, branch, w_branch, w_next, out, bias, row_index)
+    _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
+    rows, H = stream.shape
+    _need((H + 16) * 4 <= min(_max_lds_bytes(stream.device), 160 * 1024), f"the norm kernel stages one row in LDS: hidden size {H} is above its limit")
+    for t, what in ((w_branch, "w_branch"), (w_next, "w_next"), (bias, "bias")):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()), f"{what} must be float32 [{H}]")
+    if branch is not None:
+        _need(branch.dtype == torch.float32 and branch.shape == stream.shape and branch.is_contiguous() and w_branch is not None,
+              "a branch is contiguous float32 rows like the stream, with its norm's weight")
+        _need(row_index is None, "rows are picked only where no branch is added")
+    if row_index is not None:
+        _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(), "row_index must be contiguous int32")
+        rows = row_index.numel()
+    if out is None and out_dtype is not None:
+        out = torch.empty((rows, H), dtype=out_dtype, device=stream.device)
+    if out is not None:
+        _need(out.dim() == 2 and out.shape == (rows, H) and out.stride(1) == 1, f"the rows' output is [{rows}, {H}] with unit inner stride")
+    _check(_fn("float_stream.hip", "pllm_rms_sandwich",
+               signature=[c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_void_p])(
+        dtype_code(out.dtype) if out is not None else F32, _ptr(branch), _ptr(bias), _ptr(w_branch), c_float(mult), _ptr(stream), _ptr(row_index),
+        _ptr(w_next), c_float(eps), _ptr(out), out.stride(0) if out is not None else 0, rows, H, _stream()), "rms_sandwich")
+    return out
+
+
+def place_rows(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out[:, :] = x converted to out's type; x contiguous float32 [rows, hidden], out a view [rows, hidden] of wider rows."""
+    _on_gpu(x, out)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "place_rows takes contiguous float32 rows")
+    _need(out.shape == x.shape and out.stride(1) == 1, "place_rows writes rows of the same shape with unit inner stride")
+    _check(_fn("float_stream.hip", "pllm_place_rows", signature=[c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p])(
+        dtype_code(out.dtype), _ptr(x), _ptr(out), out.stride(0), x.shape[0], x.shape[1], _stream()), "place_rows")
+
+
+# ------------------------------------------------------------------------------------------- attention with normed queries and keys
+MAX_PREPARED_HEAD = 256
+
+
+def attn_prepare(proj: torch.Tensor, bias: torch.Tensor | None, conv_w: torch.Tensor | None, state: torch.Tensor | None,
+                 state_slots, seq_starts, cu_seqlens, num_seqs: int, positions: torch.Tensor, cos: torch.Tensor | None,
+                 sin: torch.Tensor | None, rot: int, interleaved: bool, eps: float, heads: int, kv_heads: int, d: int, dv: int, D: int,
+                 dtype: torch.dtype, slot_mapping: torch.Tensor | None, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None) -> torch.Tensor:
+    """From the float32 sums ``proj`` [T, >= channels] of a q/k/v product (channels = heads d + kv_heads d + kv_heads dv):
+    + ``bias``; a causal convolution over time per channel with ``conv_w`` float32 [channels, taps], whose inputs of
+    earlier steps lie in ``state[slot]`` as [taps - 1, channels] and are left there for the next step; rotary encoding
+    of the first ``rot`` elements of every q and k head; q and k heads divided by their root mean square (``eps``
+    inside the root); returns q as [T, heads * D] in ``dtype`` (heads padded with zeros to D) and writes k into
+    ``k_pages`` [pages, kv_heads, block, D] and v into ``v_pages`` [pages, kv_heads, D, block] at ``slot_mapping``."""
+    _on_gpu(proj, bias, conv_w, state, positions, cos, sin, slot_mapping, k_pages, v_pages)
+    channels = (heads + kv_heads) * d + kv_heads * dv
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= channels, f"proj: float32 [T, >= {channels}]")
+    T = proj.shape[0]
+    _need(0 < d <= D and 0 < dv <= D and D <= MAX_PREPARED_HEAD, f"head sizes {d}, {dv} padded to {D} (at most {MAX_PREPARED_HEAD})")
+    _need(rot % 2 == 0 and 0 <= rot <= d, f"rotated width {rot} of a head of {d}")
+    _need(positions.dtype == torch.int32 and positions.numel() == T and positions.is_contiguous(), "positions: int32 [T]")
+    if rot:
+        for t in (cos, sin):
+            _need(t is not None and t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(),
+                  f"rotary tables: float32 [positions, {rot // 2}]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == channels and bias.is_contiguous()), f"bias: float32 [{channels}]")
+    taps = 1
+    if conv_w is not None:
+        taps = conv_w.shape[1]
+        _need(conv_w.dtype == torch.float32 and conv_w.shape == (channels, taps) and conv_w.is_contiguous() and 1 <= taps <= MAX_CONV_TAPS,
+              f"conv weight: float32 [{channels}, taps <= {MAX_CONV_TAPS}]")
+    if taps > 1:
+        _need(state is not None, "a convolution over time needs the requests' state")
+        _check_sequences(state, state_slots, seq_starts, cu_seqlens, num_seqs)
+        _need(state.shape[1] >= channels * (taps - 1), "the convolution's inputs do not fit the state slot")
+    write = slot_mapping is not None
+    bs = 0
+    if write:
+        _need(k_pages is not None and v_pages is not None and k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous()
+              and k_pages.dtype == dtype and v_pages.dtype == dtype, "pages: contiguous, of the queries' type")
+        P, kvh, bs, dd = k_pages.shape
+        _need(kvh == kv_heads and dd == D and tuple(v_pages.shape) == (P, kvh, D, bs), "pages: k [pages, kv_heads, block, D], v [pages, kv_heads, D, block]")
+        _need(slot_mapping.dtype == torch.int32 and slot_mapping.numel() == T and slot_mapping.is_contiguous(), "slot_mapping: int32 [T]")
+    q = torch.empty((T, heads * D), dtype=dtype, device=proj.device)
+    sig = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+           c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
+    _check(_fn("attention_prepare.hip", "pllm_attn_prepare", signature=sig)(
+        dtype_code(dtype), _ptr(proj), proj.stride(0), _ptr(bias), _ptr(conv_w), taps, _ptr(state) if taps > 1 else None,
+        state.stride(0) if taps > 1 else 0, _ptr(state_slots) if taps > 1 else None, _ptr(seq_starts) if taps > 1 else None,
+        _ptr(cu_seqlens) if taps > 1 else None, num_seqs, _ptr(positions), _ptr(cos) if rot else None, _ptr(sin) if rot else None, rot,
+        int(bool(interleaved)), c_float(eps), heads, kv_heads, d, dv, D, _ptr(q), _ptr(slot_mapping) if write else None,
+        _ptr(k_pages) if write else None, _ptr(v_pages) if write else None, bs, T, _stream()), "attn_prepare")
+    return q
+
+
+def gate_heads(o: torch.Tensor, gate: torch.Tensor | None, heads: int, dv: int, D: int) -> torch.Tensor:
+    """[T, heads * dv]: the first ``dv`` elements of every head of ``o`` [T, heads * D], times sigmoid(gate[t, head]) when
+    ``gate`` (float32 [T, heads], a view with unit inner stride) is given."""
+    _on_gpu(o, gate)
+    _need(o.dim() == 2 and o.stride(1) == 1 and o.shape[1] >= heads * D and 0 < dv <= D, "gate_heads: o [T, heads * D]")
+    T = o.shape[0]
+    _need(gate is None or (gate.dtype == torch.float32 and gate.shape == (T, heads) and gate.stride(1) == 1), f"gate: float32 [{T}, {heads}]")
+    out = torch.empty((T, heads * dv), dtype=o.dtype, device=o.device)
+    _check(_fn("attention_prepare.hip", "pllm_gate_heads", signature=[c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p])(
+        dtype_code(o.dtype), _ptr(o), o.stride(0), _ptr(gate), gate.stride(0) if gate is not None else 0, _ptr(out), T, heads, dv, D, _stream()),
+        "gate_heads")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- routed experts
+MOE_TILE_ROWS = 16
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(h: torch.Tensor, router_w: torch.Tensor, correction: torch.Tensor | None, groups: int, keep: int, top: int) -> tuple:
+    """(ids int32 [T, top], weights float32 [T, top]): router outputs h router_w^T in float, softmax over all of them,
+    the ``top`` largest of score + correction among the experts of the ``keep`` best of ``groups`` groups of neighbours
+    (a group's mark: its largest corrected score), weights = the chosen experts' scores."""
+    _on_gpu(h, router_w, correction)
+    _need(h.dim() == 2 and h.stride(1) == 1, "moe_route rows: [T, width] with unit inner stride")
+    T, W = h.shape
+    n = router_w.shape[0]
+    _need(router_w.dtype == torch.float32 and router_w.shape == (n, W) and router_w.is_contiguous(), f"router: float32 [n, {W}]")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (n,) and correction.is_contiguous()), f"correction: float32 [{n}]")
+    _need(groups > 0 and n % groups == 0 and 0 < keep <= groups and 0 < top <= (n // groups) * keep,
+          f"{n} router outputs in {groups} groups, {keep} kept, {top} chosen")
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    _check(_fn("moe.hip", "pllm_moe_route", signature=[c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                                        c_void_p, c_void_p, c_void_p])(
+        dtype_code(h.dtype), _ptr(h), h.stride(0), _ptr(router_w), _ptr(correction), T, W, n, groups, keep, top, _ptr(ids), _ptr(weights),
+        _stream()), "moe_route")
+    return ids, weights
+
+
+def moe_align(ids: torch.Tensor, experts: int) -> tuple:
+    """The (token, choice) pairs of ``ids`` [T, top] whose expert is below ``experts``, sorted by expert:
+    (sorted_pair int32 [pairs], row_of_pair int32 [pairs] (-1: an expert without weights), tiles int32 [max_tiles, 3]
+    of (expert, first row, rows), rows 0 past the last tile)."""
+    _on_gpu(ids)
+    _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "ids: contiguous int32 [T, top]")
+    _need(0 < experts <= MOE_MAX_EXPERTS, f"1 to {MOE_MAX_EXPERTS} experts")
+    pairs = ids.numel()
+    max_tiles = -(-pairs // MOE_TILE_ROWS) + experts
+    sorted_pair = torch.empty(pairs, dtype=torch.int32, device=ids.device)
+    row_of_pair = torch.empty(pairs, dtype=torch.int32, device=ids.device)
+    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=ids.device)
+    _check(_fn("moe.hip", "pllm_moe_align", signature=[c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p])(
+        _ptr(ids), pairs, experts, _ptr(sorted_pair), _ptr(row_of_pair), _ptr(tiles), max_tiles, _stream()), "moe_align")
+    return sorted_pair, row_of_pair, tiles
+
+
+def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor, sorted_pair: torch.Tensor, top: int, gated: bool,
+                    activation: str = "silu") -> torch.Tensor:
+    """The experts' products over the sorted pairs.  ``gated``: rows_in [T, K] are the tokens' rows, w [experts, 2 N, K]
+    holds [gate; up] per expert, the result [pairs, N] in the rows' type is act(gate . a) * (up . a) for the pair's token.
+    Else rows_in [pairs, K] are rows in sorted order, w [experts, N, K], and the result is float32 [pairs, N]."""
+    _on_gpu(rows_in, w, tiles, sorted_pair)
+    _need(rows_in.dim() == 2 and rows_in.stride(1) == 1 and w.dim() == 3 and w.is_contiguous() and w.dtype == rows_in.dtype
+          and w.shape[2] == rows_in.shape[1], f"moe_expert_gemm shapes {tuple(rows_in.shape)} x {tuple(w.shape)}")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous(), "tiles: int32 [n, 3]")
+    pairs = sorted_pair.numel()
+    _need(sorted_pair.dtype == torch.int32 and sorted_pair.is_contiguous() and tiles.shape[0] >= -(-pairs // MOE_TILE_ROWS), "sorted pairs and their tiles")
+    K = rows_in.shape[1]
+    N = w.shape[1] // 2 if gated else w.shape[1]
+    _need(gated or rows_in.shape[0] == pairs, "the down product takes one row per pair")
+    _need(not gated or (w.shape[1] % 2 == 0 and rows_in.shape[0] * top == pairs), "the gated product takes the tokens' rows")
+    out = torch.empty((pairs, N), dtype=rows_in.dtype if gated else torch.float32, device=rows_in.device)
+    _check(_fn("moe.hip", "pllm_moe_expert_gemm", signature=[c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                                              c_void_p, c_int, c_int, c_void_p])(
+        dtype_code(rows_in.dtype), int(gated), _ptr(rows_in), rows_in.stride(0), _ptr(w), _ptr(tiles), tiles.shape[0], _ptr(sorted_pair), top, N, K,
+        _ptr(out), out.stride(0), activation_code(activation), _stream()), "moe_expert_gemm")
+    return out
+
+
+def moe_combine(expert_out: torch.Tensor, h: torch.Tensor, row_of_pair: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """float32 [T, width]: sum over a token's choices, in their order, of weight * (the pair's row of ``expert_out``
+    [pairs, width] float32, or the token's own row of ``h`` where row_of_pair is -1)."""
+    _on_gpu(expert_out, h, row_of_pair, weights)
+    T, top = weights.shape
+    W = h.shape[1]
+    _need(expert_out.dtype == torch.float32 and expert_out.shape == (T * top, W) and expert_out.is_contiguous(), f"expert outputs: float32 [{T * top}, {W}]")
+    _need(h.dim() == 2 and h.shape[0] == T and h.stride(1) == 1, "moe_combine rows: [T, width]")
+    _need(row_of_pair.dtype == torch.int32 and row_of_pair.numel() == T * top and row_of_pair.is_contiguous(), "row_of_pair: int32 [T * top]")
+    _need(weights.dtype == torch.float32 and weights.is_contiguous(), "weights: float32 [T, top]")
+    out = torch.empty((T, W), dtype=torch.float32, device=h.device)
+    _check(_fn("moe.hip", "pllm_moe_combine", signature=[c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p])(
+        dtype_code(h.dtype), _ptr(expert_out), _ptr(h), h.stride(0), _ptr(row_of_pair), _ptr(weights), T, top, W, _ptr(out), _stream()), "moe_combine")
+    return out

@@ -14,7 +14,7 @@ from collections import OrderedDict
 import numpy as np
 import torch
 
-from ..cache.block_manager import NO_PAGE
+from ..cache.block_manager import NO_PAGE, first_visible_key
 from ..cache.kv_cache import KVCacheStorage
 from .batch import GroupView, StepContext, StepEntry
 
@@ -172,7 +172,7 @@ class ModelRunner:
                     raise StepError(f"request {e.request_id!r}: {len(table)} pages in group {name!r}, "
                                     f"{k_lens[s]} positions need {need}")
                 # Pages a query of this step can see: from the first key inside the window on.
-                first_key = max(0, e.start - cs.window + 1) if cs.window > 0 else 0
+                first_key = first_visible_key(cs.kind, cs.window, e.start)
                 known = self._checked_rows.get((e.request_id, name)) if e.table_version is not None else None
                 if known is not None and known[0] == (e.table_version, need, first_key // bs):
                     shown = known[1]                                 # this table was checked and converted in an earlier step
@@ -375,7 +375,7 @@ class ModelRunner:
                     raise StepError(f"request {e.request_id!r} has no block table for cache group {name!r}")
                 n = min(len(table), fixed)
                 row = np.asarray(table[:n], dtype=np.int64)
-                first_key = max(0, e.start - cs.window + 1) if cs.window > 0 else 0
+                first_key = first_visible_key(cs.kind, cs.window, e.start)
                 live = row[first_key // bs:]
                 if live.size and (live.min() < 0 or live.max() >= num_pages):
                     raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")

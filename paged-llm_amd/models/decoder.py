@@ -26,6 +26,8 @@ class DecoderModel:
             block = registry.build("block", layer.block, env)
             block.build_parts(layer.parts, env)
             self.blocks.append(block)
+        # operations on the stream between layers, which schedule steps name as their entry
+        self.stream_ops = [registry.build("stream_op", op.part, env) for op in spec.stream_ops]
         self.final_norm = registry.build("norm", spec.final_norm, env)
         self.head = registry.build("head", spec.head, env)
         self._ready = False
@@ -36,6 +38,8 @@ class DecoderModel:
         out = {tensor_name(s.embedding_name, n): w for n, w in self.embedding.weight_specs().items()}
         for layer, block in zip(s.layers, self.blocks):
             out.update({tensor_name(layer.name, n): w for n, w in block.weight_specs().items()})
+        for op, part in zip(s.stream_ops, self.stream_ops):
+            out.update({tensor_name(op.name, n): w for n, w in part.weight_specs().items()})
         out.update({tensor_name(s.final_norm_name, n): w for n, w in self.final_norm.weight_specs().items()})
         out.update({tensor_name(s.head_name, n): w for n, w in self.head.weight_specs().items()})
         return out
@@ -49,7 +53,8 @@ class DecoderModel:
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
         s = self.spec
-        for prefix, part in [(s.embedding_name, self.embedding), (s.final_norm_name, self.final_norm), (s.head_name, self.head)]:
+        outside = [(s.embedding_name, self.embedding), (s.final_norm_name, self.final_norm), (s.head_name, self.head)]
+        for prefix, part in outside + [(op.name, part) for op, part in zip(s.stream_ops, self.stream_ops)]:
             own = name_under(prefix, name)
             if own is not None and own in part.weight_specs():
                 return part.assign(own, tensor)
@@ -63,6 +68,8 @@ class DecoderModel:
         self.embedding.finalize()
         for b in self.blocks:
             b.finalize()
+        for op in self.stream_ops:
+            op.finalize()
         self.final_norm.finalize()
         self.head.finalize()
         if getattr(self.head, "tied", False):
@@ -95,7 +102,8 @@ class DecoderModel:
     def graph_capturable(self, prompts: bool = False) -> bool:
         """True when every layer's parts only launch kernels (no host reads of device data, no Python-side
         state): a decode step (``prompts``: also a step with prompt portions) can then be captured into a HIP graph."""
-        return all(b.graph_capturable(prompts) for b in self.blocks)
+        flag = "graph_capturable_prompts" if prompts else "graph_capturable"
+        return all(b.graph_capturable(prompts) for b in self.blocks) and all(getattr(op, flag, False) for op in self.stream_ops)
 
     def graph_step_arrays(self, layout) -> dict:
         """Host-made integer arrays the layers' parts need for a replayed step of that layout (equal keys are one array)."""
@@ -112,9 +120,20 @@ class DecoderModel:
         x = self.embedding.forward(ctx.input_ids)
         delta = None
         schedule = self.spec.schedule
+        # the embedding's output for the stream operations: a tensor of its own where the layers add to the stream in place
+        x0 = None
+        if self.stream_ops:
+            x0 = self.embedding.forward(ctx.input_ids) if getattr(self.embedding, "float_stream", False) else x
         last_takes_partial = bool(getattr(self.final_norm, "accepts_partial_sums", False))
         for pos, step in enumerate(schedule):
             block = self.blocks[step.layer]
+            if step.entry is not None:
+                if delta is not None:
+                    raise RuntimeError("a stream operation takes the stream with every sum done")
+                x = self.stream_ops[step.entry].forward(x, x0, ctx)
+            # the norm that reads the stream next, for a block that can compute its rows while it forms the stream's last sum
+            following = schedule[pos + 1] if pos + 1 < len(schedule) else None
+            ctx.next_entry_norm = (self.blocks[following.layer].entry_norm() if following is not None and following.entry is None else None)
             cache = None
             if block.cache_spec() is not None:
                 owner = pos if step.cache_from is None else step.cache_from

@@ -70,19 +70,20 @@ class CacheSpec:
     widths ...).  The cache storage allocates ``[pages, *page shape]`` per named tensor and hands them to the mixer
     by name; the cache manager only counts pages.  Layers with equal specs share a group of pages (one block table
     per request and group)."""
-    kind: str                 # "full": all positions;  "window": only the last `window` positions
+    kind: str                 # "full": all positions;  "window": only the last `window` positions;
+                              # "chunk": only the positions of the newest block of `window` positions (blocks counted from 0)
     tensors: tuple            # of PageTensor
-    window: int = 0           # > 0 for kind "window"
+    window: int = 0           # > 0 for the kinds "window" and "chunk"
 
     def __post_init__(self):
-        if self.kind not in ("full", "window") or (self.kind == "window") != (self.window > 0):
-            raise ValueError(f"cache kind {self.kind!r} with window {self.window}: \"full\", or \"window\" with a window > 0")
+        if self.kind not in ("full", "window", "chunk") or (self.kind != "full") != (self.window > 0):
+            raise ValueError(f"cache kind {self.kind!r} with window {self.window}: \"full\", or \"window\" / \"chunk\" with a size > 0")
         names = [t.name for t in self.tensors]
         if not names or len(set(names)) != len(names):
             raise ValueError(f"a cache spec names at least one page tensor, each once; got {names}")
 
     def group_name(self) -> str:
-        base = f"{self.kind}{self.window if self.kind == 'window' else ''}"
+        base = f"{self.kind}{self.window if self.kind != 'full' else ''}"
         def one(t):
             dims = "x".join("B" if d == BLOCK else str(d) for d in t.shape)
             return f"{t.name}{dims}" + (f":{str(t.dtype).split('.')[-1]}" if t.dtype is not None else "")
@@ -201,6 +202,17 @@ class Mixer(Part):
         raise NotImplementedError
 
 
+class StreamOp(Part):
+    """An operation on the residual stream between layers: ``forward(x, x0, ctx) -> x`` with x the stream as the layer
+    before left it (every sum done) and x0 the embedding's output.  It returns the stream that the next layer reads
+    and adds to (a tensor of its own: x0 is never written to)."""
+    graph_capturable = True
+    graph_capturable_prompts = True
+
+    def forward(self, x: torch.Tensor, x0: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         raise NotImplementedError
@@ -255,6 +267,11 @@ class Block(Part):
         for part in self.parts.values():
             out.update(part.graph_step_arrays(layout))
         return out
+
+    def entry_norm(self):
+        """The norm that first reads the stream in this block, when whoever leaves the stream may compute that norm's
+        rows in the kernel that forms the stream's last sum (``ctx.next_entry_norm``); None: the block norms for itself."""
+        return None
 
     def accepts_partial_delta(self) -> bool:
         """Whether the ``delta`` this block is handed may be float partial sums [ranges, rows, hidden] instead of rows

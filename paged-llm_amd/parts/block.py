@@ -93,3 +93,64 @@ class BranchNormBlock(Block):
 
 
 register_block("branch_norm", BranchNormBlock)
+
+
+class SandwichNormBlock(Block):
+    """A block with a norm in front of and behind every branch, over a residual stream kept in float:
+
+        x <- x + m * norm_b(mixer(norm_a(x)));   x <- x + m * norm_d(feed_forward(norm_c(x)))    (the second line only with a feed-forward)
+
+    The branches' last products leave float rows (``ctx.float_branch``); one kernel norms them, adds them times m to the
+    stream in place and computes, from the row it still holds, the rows that whoever reads the stream next wants: this
+    block's next norm, or the first norm of the layer that follows (``ctx.next_entry_norm``, set by the model), which
+    travel beside the stream in ``ctx.launch_cache``.  A branch may hand a bias of its last product to that kernel
+    (``output_bias`` of the part) instead of adding it itself.
+
+    params: ``residual_mult`` (m), ``feed_forward`` (False: the mixer alone), and the roles' prefixes in tensor names."""
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "mixer_out_norm": "norm",
+             "feed_forward_norm": "norm", "feed_forward": "feed_forward", "feed_forward_out_norm": "norm"}
+    _ROWS = "sandwich_rows"
+
+    def __init__(self, params: dict, env):
+        self.has_feed_forward = bool(params.get("feed_forward", True))
+        if not self.has_feed_forward:
+            self.ROLES = {r: f for r, f in self.ROLES.items() if not r.startswith("feed_forward")}
+        super().__init__({k: v for k, v in params.items() if k in self.ROLES and isinstance(v, str)}, env)
+        self.mult = float(params.get("residual_mult", 1.0))
+        self.dtype = env.dtype
+
+    def entry_norm(self):
+        return self.parts["mixer_norm"]
+
+    def _entry_rows(self, x, ctx):
+        """norm_a(x) in the compute type: what the kernel that last wrote x left for this norm, or computed now."""
+        norm = self.parts["mixer_norm"]
+        held = ctx.launch_cache.get(self._ROWS)
+        if held is not None and held[0] is x and held[1] is norm:
+            return held[2]
+        return norm.forward(x)
+
+    def forward(self, x, delta, ctx, cache, state):
+        p = self.parts
+        if delta is not None:
+            raise RuntimeError("a block over a float stream takes the stream with every sum done")
+        if x.dtype != torch.float32:
+            raise RuntimeError("this block keeps its residual stream in float32 (an embedding with float_stream)")
+        after = getattr(ctx, "next_entry_norm", None)
+        ctx.partial_sums_ok, ctx.float_branch = False, True
+        ctx.branch_bias_taken = True          # a bias of a branch's last product is added by the kernel that norms the branch
+        a = p["mixer"].forward(self._entry_rows(x, ctx), ctx, cache, state)
+        bias = getattr(p["mixer"], "output_bias", None)
+        if self.has_feed_forward:
+            h = p["mixer_out_norm"].add_to(x, a, self.mult, bias=bias, then=p["feed_forward_norm"])
+            m = p["feed_forward"].forward(h, ctx)
+            a, bias, last = m, getattr(p["feed_forward"], "output_bias", None), p["feed_forward_out_norm"]
+        else:
+            last = p["mixer_out_norm"]
+        rows = last.add_to(x, a, self.mult, bias=bias, then=after, want_rows=after is not None)
+        ctx.launch_cache[self._ROWS] = (x, after, rows) if after is not None else None
+        ctx.float_branch = ctx.branch_bias_taken = False
+        return x, None
+
+
+register_block("sandwich_norm", SandwichNormBlock)

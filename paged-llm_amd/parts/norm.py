@@ -89,26 +89,46 @@ class RMSNorm(Norm):
     accepts_partial_sums = True
 
     def __init__(self, params: dict, env: BuildEnv):
+        """params: ``eps``; ``size`` (default: the model's width); ``weight_name`` (the weight's own name under the part's
+        prefix, default "weight"; "" is the prefix itself); ``unit_offset`` (the checkpoint stores w - 1: the factor
+        applied is 1 + what is stored, formed in float when the weight arrives)."""
         self.eps = float(params["eps"])
         self.size = int(params.get("size", env.hidden_size))
-        self.device = env.device
+        self.weight_name = params.get("weight_name", "weight")
+        self.unit_offset = bool(params.get("unit_offset", False))
+        self.dtype, self.device = env.dtype, env.device
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.size,), role="vector", init="ones")}
+        return {self.weight_name: WeightSpec((self.size,), role="vector", init="zeros" if self.unit_offset else "ones")}
 
     def assign(self, name, tensor):
-        if name != "weight":
+        if name != self.weight_name:
             raise KeyError(name)
-        self.weight = tensor.to(device=self.device, dtype=torch.float32).contiguous()
+        w = tensor.to(device=self.device, dtype=torch.float32)
+        self.weight = (w + 1.0 if self.unit_offset else w).contiguous()
 
     def forward(self, x, row_index=None):
+        if x.dtype == torch.float32 and self.dtype != torch.float32:        # rows of a float stream, normed into the compute type
+            return ops.rms_sandwich(x, None, None, 0.0, self.eps, w_next=self.weight, out_dtype=self.dtype, row_index=row_index)
         return ops.rmsnorm(x, self.weight, self.eps, None, row_index)
+
+    def add_to(self, stream: torch.Tensor, branch: torch.Tensor, mult: float = 1.0, bias: torch.Tensor | None = None,
+               then: "RMSNorm | None" = None, out: torch.Tensor | None = None, want_rows: bool = True):
+        """stream += mult * norm(branch + bias), in place and in float (a block that norms what its branches return).
+        Returns the new stream's rows in the compute type for whoever reads them next, computed in the same kernel:
+        normed by ``then`` (the reader's own norm), or as they are; into ``out`` when given; None unless ``want_rows``."""
+        if then is not None and (then.eps != self.eps or then.size != self.size):
+            raise ValueError("the norm behind the sum shares this norm's width and eps")
+        return ops.rms_sandwich(stream, branch, self.weight, mult, self.eps, w_next=then.weight if then is not None else None,
+                                out=out, out_dtype=self.dtype if want_rows and out is None else None, bias=bias)
 
     def add_norm(self, x, delta, row_index=None, write_residual=True):
         return ops.rmsnorm(x, self.weight, self.eps, delta, row_index, write_residual)
 
-    def pending(self, x, delta=None, row_index=None, write_residual=True) -> PendingNorm:
+    def pending(self, x, delta=None, row_index=None, write_residual=True):
+        if x.dtype == torch.float32 and self.dtype != torch.float32 and delta is None:
+            return Norm.pending(self, x, None, row_index, write_residual)       # rows of a float stream: normed at once, into the compute type
         return PendingNorm(self.weight, self.eps, x, delta, row_index, write_residual)
 
 

@@ -20,9 +20,10 @@ POSITION_ENCODINGS: dict = {}
 BLOCKS: dict = {}
 EMBEDDINGS: dict = {}
 HEADS: dict = {}
+STREAM_OPS: dict = {}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position_encoding": POSITION_ENCODINGS,
-           "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS}
+           "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS, "stream_op": STREAM_OPS}
 
 
 @dataclass
@@ -55,6 +56,7 @@ def register_position_encoding(kind: str, cls) -> None: _register(POSITION_ENCOD
 def register_block(kind: str, cls) -> None: _register(BLOCKS, kind, cls)
 def register_embedding(kind: str, cls) -> None: _register(EMBEDDINGS, kind, cls)
 def register_head(kind: str, cls) -> None: _register(HEADS, kind, cls)
+def register_stream_op(kind: str, cls) -> None: _register(STREAM_OPS, kind, cls)
 
 
 def build(family: str, spec: PartSpec, env: BuildEnv):

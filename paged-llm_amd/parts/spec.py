@@ -32,7 +32,7 @@ class WeightSpec:
     """
     shape: tuple
     role: str = "matrix"
-    # For the random-weights mode: "normal" (std 0.02) or "ones".
+    # For the random-weights mode: "normal" (std 0.02), "ones", or "zeros" (a norm weight stored as w - 1).
     init: str = "normal"
 
 
@@ -54,9 +54,20 @@ class ScheduleStep:
 
     A layer named by several steps shares its weights between them; each step still owns a
     cache and a state of its own, because what it sees differs.  ``cache_from`` names an earlier
-    step whose cache this step's mixer reads instead of writing one."""
+    step whose cache this step's mixer reads instead of writing one.  ``entry`` names a stream operation of the model
+    (an index into ``ModelSpec.stream_ops``) that acts on the residual stream right before this step's layer."""
     layer: int
     cache_from: int | None = None
+    entry: int | None = None
+
+
+@dataclass
+class StreamOpSpec:
+    """An operation on the residual stream between layers (family "stream_op" of the part registry), with the prefix
+    of its tensor names in the checkpoint.  Schedule steps name it by its index; one operation may stand in front of
+    several steps (the same weights each time)."""
+    name: str
+    part: PartSpec
 
 
 @dataclass
@@ -69,6 +80,8 @@ class ModelSpec:
     head: PartSpec
     # The order in which layers run; empty = every layer once, in order.
     schedule: list[ScheduleStep] = field(default_factory=list)
+    # Operations on the residual stream that schedule steps name as their ``entry``.
+    stream_ops: list = field(default_factory=list)      # of StreamOpSpec
     # Prefixes of the tensor names of the parts outside the layers (the architecture says them: "" is no default
     # that fits any family of checkpoints).
     embedding_name: str = ""
@@ -90,6 +103,8 @@ class ModelSpec:
         for pos, step in enumerate(self.schedule):
             if not 0 <= step.layer < len(self.layers):
                 raise ValueError(f"schedule step {pos} names layer {step.layer}, the model has {len(self.layers)}")
+            if step.entry is not None and not 0 <= step.entry < len(self.stream_ops):
+                raise ValueError(f"schedule step {pos} names stream operation {step.entry}, the model has {len(self.stream_ops)}")
             src = step.cache_from
             if src is not None:
                 if not 0 <= src < pos:

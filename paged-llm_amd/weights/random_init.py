@@ -35,8 +35,8 @@ def draw_weights(weight_specs: dict, seed: int, stored: torch.dtype = torch.floa
         ws = weight_specs[name]
         if ws.role == "int":
             raise NotImplementedError("random integer tables")
-        if ws.init == "ones":
-            t = torch.ones(ws.shape, dtype=torch.float32)
+        if ws.init in ("ones", "zeros"):                       # ("zeros": a norm weight stored as w - 1)
+            t = torch.ones(ws.shape, dtype=torch.float32) if ws.init == "ones" else torch.zeros(ws.shape, dtype=torch.float32)
             if norm_jitter:
                 t = t + 0.1 * torch.randn(ws.shape, generator=gen, dtype=torch.float32)
         else:
