@@ -98,6 +98,56 @@ def run_gudutar(dtype: str, context: int, steps: int, warmup: int, widths=(1024,
     return out
 
 
+def mutapel_config(width: int, vocab: int, window: int = 1024, block: int = 2048) -> dict:
+    """Mutapel at sizes that resemble a real model's layers: eight layers of which the middle four run twice (twelve
+    layer runs), the two attention layers by turns.  Heads of 64 elements as the Llama model beside it has, one key head
+    per eight heads; the layer with a sliding window sees ``window`` positions, the one with blocks convolves over four
+    taps and sees its block of ``block`` positions.  Every layer routes each token to 4 of 30 experts and 2 pass-through
+    ones (4 groups of 8, the best 2 kept); an expert is 11/16 of the width wide, so the four chosen ones do the work of
+    the dense feed-forward of 2.75 times the width that the Llama model has."""
+    heads = width // 64
+    kv = max(1, heads // 8)
+    win = {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 64, "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}, "scale": 0.125}
+    blk = dict(win, conv=4, mask={"size": block})
+    mlp = {"kind": "moe", "expert": {"ff": 11 * width // 16},
+           "router": {"experts": 30, "identity": 2, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    layers = [{"type": ("attention_2", "attention")[i % 2], "mixer": dict((win, blk)[i % 2]), "mlp": dict(mlp)} for i in range(8)]
+    return {"architecture": "Mutapel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "layers": layers,
+            "loop": {"start": 2, "stop": 6, "times": 2}, "max_positions": 4096, "torch_dtype": "bfloat16"}
+
+
+def run_mutapel(dtype: str, context: int, steps: int, warmup: int, widths=(1024, 2048)) -> dict:
+    """Prefill (one prompt of 512 and of 2048 tokens in one step) and decode (1, 8 and 64 requests at ``context``) of
+    Mutapel beside the Llama decoder at the same width, number of layer runs, heads, active feed-forward width and
+    vocabulary (random weights).  Mutapel holds 30 experts where the Llama model holds one feed-forward, so it is far
+    heavier in weights; per token it multiplies by as many."""
+    import torch
+    out = {}
+    for width in widths:
+        models = {
+            "mutapel": mutapel_config(width, 32000),
+            "llama": dict(TINYLLAMA, num_hidden_layers=12, hidden_size=width, num_attention_heads=width // 64,
+                          num_key_value_heads=max(1, width // 512), head_dim=64, intermediate_size=11 * width // 4, torch_dtype=dtype),
+        }
+        for name, cfg in models.items():
+            row = {}
+            with tempfile.TemporaryDirectory() as folder:
+                engine = make_engine(cfg, folder, dtype, 64, context)
+                for tokens in (512, PREFILL_TOKENS):
+                    t = time_prefill(engine, tokens, seed=100 + tokens, repeats=4)
+                    row[f"prefill_{tokens}_ms"] = round(t * 1e3, 3)
+                    row[f"prefill_{tokens}_tok_per_s"] = round(tokens / t, 1)
+                for batch in (1, 8, 64):
+                    sec, _ = time_decode(engine, batch, context, steps, warmup, seed=batch)
+                    row[f"decode_b{batch}_ms"] = round(sec * 1e3, 4)
+                    row[f"decode_b{batch}_tok_per_s"] = round(batch / sec, 1)
+                row["weights_millions"] = round(sum(_weights_of(engine.model)) / 1e6, 1)
+                del engine
+                torch.cuda.empty_cache()
+            out[f"{name}_w{width}"] = row
+    return out
+
+
 def _weights_of(model):
     """Numbers of elements of the tensors the model declares (what a checkpoint of it holds)."""
     out = []
@@ -620,6 +670,8 @@ def main() -> int:
     ap.add_argument("--context-sweep", default=None, metavar="N,N,...", help="decode at --batch requests (and prefill up to 8192) at each of these contexts")
     ap.add_argument("--gudutar", action="store_true", help="prefill and decode of the Gudutar decoder (state-space, retention and "
                     "latent-attention layers) at two widths beside the Llama decoder of the same width and depth, instead")
+    ap.add_argument("--mutapel", action="store_true", help="prefill and decode of the Mutapel decoder (windowed and blocked attention with "
+                    "normed queries and keys, routed experts) beside a Llama decoder of the same width and depth, and nothing else")
     ap.add_argument("--kernels", action="store_true", help="every kernel of a decode step and of a prompt step on its own, with its fraction")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -641,6 +693,11 @@ def main() -> int:
         print(json.dumps({"metric": "Gudutar beside the Llama decoder at equal width, depth and vocabulary (random weights): prefill and decode",
                           "dtype": short, "context": args.context,
                           "models": run_gudutar(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2))}))
+        return 0
+    if args.mutapel:
+        print(json.dumps({"metric": "Mutapel beside the Llama decoder at equal width, layer runs, heads and vocabulary (random weights): prefill and decode",
+                          "dtype": short, "context": args.context,
+                          "models": run_mutapel(args.dtype, args.context, max(16, args.steps // 2), max(4, args.warmup // 2))}))
         return 0
     if args.workload == "ragged64":
         print(json.dumps({"metric": f"output tokens/s, 64 ragged requests at once, prompts 64-2048 tokens, 256 generated each ({model_name}, random weights)",

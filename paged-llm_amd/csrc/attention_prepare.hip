@@ -20,7 +20,7 @@ constexpr int kPrepMaxHead = 256;
 constexpr int kPrepMaxTaps = 16;
 
 // proj      [tokens, ld] float: columns [q heads * d | kv heads * d | kv heads * dv | ...]
-// bias      [channels] float or null;  conv_w [channels, taps] float or null (taps <= 1: no convolution)
+// bias      [channels] float or null;  conv_w [channels, taps] float or null (null: no convolution)
 // state     [slots][taps - 1][channels] float, oldest first: the projected values (with bias) of the tokens before
 //           this step's; a sequence with seq_starts == 0 has zeros there whatever the slot holds.
 // q_out     [tokens, heads * D];  k_pages [pages, kv heads, block, D];  v_pages [pages, kv heads, D, block]
@@ -73,6 +73,7 @@ __global__ __launch_bounds__(64) void attn_prepare_kernel(
         }
       } else {
         v = proj[(size_t)tok * ld + c] + b;
+        if (conv_w) v *= conv_w[c];                              // one tap: a factor per channel
       }
     }
     x[r] = v;

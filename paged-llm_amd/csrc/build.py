@@ -146,9 +146,9 @@ def load_library(source: str, defines: dict | None = None) -> ctypes.CDLL:
 COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "decode_linear.hip",
                   "attention_noalloc.hip", "stream_linear.hip", "float_stream.hip", "recurrent.hip", "latent_attention.hip", "attention_prepare.hip", "moe.hip"]
 # Head sizes whose attention library a full build makes (others are compiled at first use).
-USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
+USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 256)
 # ... and those whose attention library with further score terms in its loops (-DSCORE_TERMS=1) it makes as well.
-SCORE_TERMS_HEAD_DIMS = (16, 32, 64, 128)
+SCORE_TERMS_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 144)
 
 
 def all_targets() -> list[tuple[str, dict]]:

@@ -29,7 +29,7 @@ MASKS = ("full", "window", "chunk")
 class NormedAttention(Mixer):
     """params: ``heads``, ``kv_heads``, ``key_dim``, ``value_dim``, ``scale``, ``eps`` (of the q/k norm), ``position`` (a
     rotary spec or None), ``mask`` ("full", "window" or "chunk") with ``mask_size``, ``conv`` (taps of the convolution
-    over time; 0 or 1: none), ``bias`` (q, k, v and the output product have biases), ``sinks`` (a logit per head in the
+    over time; 0: none), ``bias`` (q, k, v and the output product have biases), ``sinks`` (a logit per head in the
     softmax's sum), ``head_gate`` (a gate per head from the mixer's input).  Tensors (under the part's prefix): ``q``,
     ``k``, ``v``, ``o``; ``q.b``, ``k.b``, ``v.b``, ``o.b``; ``q.conv``, ``k.conv``, ``v.conv`` [channels, taps];
     ``sink`` [heads]; ``g`` [heads, width]."""
@@ -42,6 +42,7 @@ class NormedAttention(Mixer):
         self.d, self.dv = int(params["key_dim"]), int(params["value_dim"])
         self.scale, self.eps = float(params["scale"]), float(params["eps"])
         self.mask, self.mask_size = params.get("mask") or "full", int(params.get("mask_size") or 0)
+        self.has_conv = int(params.get("conv") or 0) >= 1
         self.taps = max(1, int(params.get("conv") or 1))
         self.bias, self.has_sinks, self.head_gate = bool(params.get("bias")), bool(params.get("sinks")), bool(params.get("head_gate"))
         if self.heads % self.kv_heads:
@@ -71,7 +72,7 @@ class NormedAttention(Mixer):
         if self.bias:
             specs.update({"q.b": WeightSpec((q,), role="vector"), "k.b": WeightSpec((k,), role="vector"), "v.b": WeightSpec((v,), role="vector"),
                           "o.b": WeightSpec((self.hidden,), role="vector")})
-        if self.taps > 1:
+        if self.has_conv:
             specs.update({f"{n}.conv": WeightSpec((c, self.taps), role="vector") for n, c in (("q", q), ("k", k), ("v", v))})
         if self.has_sinks:
             specs["sink"] = WeightSpec((self.heads,), role="vector")
@@ -92,7 +93,7 @@ class NormedAttention(Mixer):
         if self.bias:
             self.b_in = torch.cat([w.pop(n) for n in ("q.b", "k.b", "v.b")]).contiguous()
             self.output_bias = w.pop("o.b")           # added by whoever norms the mixer's float output (the block's kernel)
-        if self.taps > 1:
+        if self.has_conv:
             self.conv_w = torch.cat([w.pop(n) for n in ("q.conv", "k.conv", "v.conv")], dim=0).contiguous()
         terms = ops.ScoreTerms(0.0, None, w.pop("sink") if self.has_sinks else None)
         self.terms = terms if terms.any() else None

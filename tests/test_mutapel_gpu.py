@@ -1,0 +1,610 @@
+"""Mutapel in the engine against the plain implementation under tests/plain/: each mechanism alone, whole prompts,
+token-by-token decoding, portions down to two tokens, unequal requests in one batch with pages and state slots used
+again, keys far back, at page borders and on either side of a window's and a block's edge (with weights made so that
+one score stands out), logits in the softmax's denominator, the first tokens of a sequence, long decoding, sizes of
+several kinds, and greedy generation through ``LLMEngine``."""
+
+import copy
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers
+from tests.helpers import TraceBuilder
+from tests.mutapel_configs import ALONE, MUTA_A, MUTA_B, MUTA_C, _blocks, _layer, _moe, _window, model
+from tests.plain import mutapel_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {"A": MUTA_A, "B": MUTA_B, "C": MUTA_C, **ALONE}
+TOL = {"float32": 3e-5, "bfloat16": 6e-2}
+
+
+def write_folder(path, cfg, seed, stored, edit=None):
+    """A model folder with random weights (stored norm weights near zero, everything else normal with the width's
+    scale); ``edit(tensors)`` may change them before they are stored."""
+    from safetensors.torch import load_file, save_file
+    from paged_llm_amd.weights import write_random_model
+    folder = write_random_model(str(path), cfg, seed=seed, dtype=stored, std=cfg["width"] ** -0.5, norm_jitter=True)
+    if edit is not None:
+        file = os.path.join(folder, "model.safetensors")
+        tensors = load_file(file)
+        edit(tensors)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, file)
+    return folder
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+
+    def get(name, stored):
+        if (name, stored) not in made:
+            made[name, stored] = write_folder(tmp_path_factory.mktemp(f"mutapel_{name}_{stored}"), CONFIGS[name],
+                                              seed=23 + len(name), stored=stored)
+        return made[name, stored]
+    return get
+
+
+_plain_cache: dict = {}
+
+
+def plain_logits(folder, tokens):
+    key = (folder, tuple(tokens))
+    if key not in _plain_cache:
+        _plain_cache[key] = plain.forward(plain.read_config(folder), plain.load_weights(folder), list(tokens)).numpy()
+    return _plain_cache[key]
+
+
+def session_for(folder, dtype, max_tokens, **kw):
+    from paged_llm_amd.engine.replay import ReplaySession
+    return ReplaySession(folder, dtype, max_tokens, None, **kw)
+
+
+_noise_cache: dict = {}
+
+
+def rounding_scale(folder, tokens):
+    """Per position: how far the plain logits move (root mean square over four draws of ``helpers.worst``) when every
+    product's rows and result carry the relative error of bfloat16 rounding.  Positions differ in how much rounding
+    moves them (a softmax between two near-equal scores, an expert chosen by a hair), so a bfloat16 result is judged
+    against its own position's scale."""
+    key = (folder, tuple(tokens))
+    if key not in _noise_cache:
+        exact = plain_logits(folder, tokens)
+        cfg, weights = plain.read_config(folder), plain.load_weights(folder)
+        sq = np.zeros(len(tokens))
+        for seed in range(4):
+            with plain.rounding_noise(seed):
+                moved = plain.forward(cfg, weights, list(tokens)).numpy()
+            sq += (np.abs(moved - exact).max(axis=1) / np.abs(exact).max(axis=1)) ** 2
+        _noise_cache[key] = np.sqrt(sq / 4)
+    return _noise_cache[key]
+
+
+_exact_cache: dict = {}
+
+
+def float32_scale(folder, tokens):
+    """Per position: how far the plain implementation in float32 is from itself in float64."""
+    key = (folder, tuple(tokens))
+    if key not in _exact_cache:
+        exact = plain.forward(plain.read_config(folder), plain.load_weights(folder), list(tokens), dtype=torch.float64).numpy()
+        _exact_cache[key] = np.abs(plain_logits(folder, tokens) - exact).max(axis=1) / np.abs(exact).max(axis=1)
+    return _exact_cache[key]
+
+
+def bound_at(folder, tokens, pos, dtype):
+    """What a row may differ by: in float32 3e-5, or 5 times the plain implementation's own float32 error at that
+    position if that is more; in bfloat16 4 times the position's rounding scale, at least 3e-2."""
+    if dtype == "float32":
+        return max(TOL[dtype], 5.0 * float(float32_scale(folder, tokens)[pos]))
+    return max(3e-2, 4.0 * float(rounding_scale(folder, tokens)[pos]))
+
+
+def check(got: dict, folder, reqs: dict, dtype, narrow=False):
+    """Every row within its bound in float32.  In bfloat16, models without routed experts: no row beyond twice its
+    bound, at most one in fifty beyond it, and the median error below 2.5e-2.  In bfloat16 with routed experts the
+    choice of an expert is a discrete step: where two corrected scores are closer than the compute type's rounding of
+    the rows in front of them, the engine and the plain implementation may choose differently, and what that changes
+    reaches every later position through keys and values.  With hundreds of choices in a request some are that close
+    whatever the tokens, so those rows are judged as a whole: the median error below 5e-2 and at most half of the rows
+    beyond their bound (a fault in a kernel moves most rows by their whole size; float32 runs of the same models, where
+    every row is held to 3e-5, and ``test_experts_with_a_decisive_choice`` are the sharp tests of the experts' kernels)."""
+    want = {rid: plain_logits(folder, toks) for rid, toks in reqs.items()}
+    routed = any(l.get("mlp") for l in plain.read_config(folder)["layers"])
+    ratios, errs = {}, []
+    for (rid, pos), row in got.items():
+        err = helpers.worst(row, want[rid][pos])
+        errs.append(err)
+        ratios[rid, pos] = err / bound_at(folder, reqs[rid], pos, dtype)
+    worst_at = max(ratios, key=ratios.get)
+    over = sum(1 for r in ratios.values() if r > 1.0)
+    said = f"{worst_at}: {ratios[worst_at]:.3g} of its bound (median error {np.median(errs):.3g}), {over} of {len(ratios)} rows over"
+    if dtype == "float32":
+        assert ratios[worst_at] <= 1.0, said
+    elif routed:
+        assert np.median(errs) <= 5e-2 and over <= len(ratios) // 2, said
+    else:
+        # (narrow: models a few dozen channels wide, whose rows move more under rounding and whose few draws of the
+        #  yardstick say less: twice the allowances)
+        most, middle = (4.0, 5e-2) if narrow else (2.0, 2.5e-2)
+        assert ratios[worst_at] <= most and over <= max(1, len(ratios) // 50) and np.median(errs) <= middle, said
+
+
+def whole(reqs):
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        trace.step([(rid, toks, "all")], end=[rid])
+    return trace
+
+
+def prompt_then_single(rid, toks, cut, want="all"):
+    trace = TraceBuilder().step([(rid, toks[:cut], want)], end=[rid] if cut == len(toks) else [])
+    for i in range(cut, len(toks)):
+        trace.step([(rid, toks[i:i + 1], "all")], end=[rid] if i == len(toks) - 1 else [])
+    return trace
+
+
+def stored_as(dtype):
+    return "float32" if dtype == "float32" else "bfloat16"
+
+
+# --------------------------------------------------------------------------- each mechanism alone, and whole models
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_whole_prompts(folders, name, dtype):
+    folder = folders(name, stored_as(dtype))
+    vocab = CONFIGS[name]["vocab"]
+    reqs = {"p1": helpers.random_tokens(1, vocab, 1), "p5": helpers.random_tokens(5, vocab, 2), "p70": helpers.random_tokens(70, vocab, 3)}
+    got = helpers.replay_in_process(session_for(folder, dtype, 128), whole(reqs))
+    assert len(got) == 76
+    check(got, folder, reqs, dtype, narrow=name == "B")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "blocks", "window", "repeated"])
+def test_prompt_then_token_by_token(folders, name, dtype):
+    """A prompt in one step and then single tokens: pages, the convolution's rows in the state slot, windows and blocks
+    whose edges pass among decoded tokens."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(75, CONFIGS[name]["vocab"], 7)
+    session = session_for(folder, dtype, 128)
+    check(helpers.replay_in_process(session, prompt_then_single("r", toks, 13)), folder, {"r": toks}, dtype, narrow=name == "B")
+    assert any(key[0] != "prompt" for key in session.runner._graphs), "single-token steps are replayed from graphs"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_token_by_token_from_the_first(folders, name, dtype):
+    """No prompt step at all: the first tokens meet the convolution's zeros, a softmax over one key and a logit without
+    a key, and blocks and windows of one position."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(12, CONFIGS[name]["vocab"], 8)
+    check(helpers.replay_in_process(session_for(folder, dtype, 64), prompt_then_single("r", toks, 1)), folder, {"r": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("sizes", [[2], [3, 2, 7], [16, 1, 17, 2, 31], [64, 5]])
+def test_portions(folders, name, dtype, sizes):
+    """Prompts cut into portions of several sizes, down to two tokens (shorter than the convolution's reach), cut in
+    the middle of pages, windows and blocks."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(97, CONFIGS[name]["vocab"], 9)
+    trace, at, k = TraceBuilder(), 0, 0
+    while at < len(toks):
+        n = min(sizes[k % len(sizes)], len(toks) - at)
+        trace.step([("r", toks[at:at + n], "all")], end=["r"] if at + n == len(toks) else [])
+        at, k = at + n, k + 1
+    check(helpers.replay_in_process(session_for(folder, dtype, 128), trace), folder, {"r": toks}, dtype, narrow=name == "B")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_logits_do_not_depend_on_the_cut(folders, name, dtype):
+    """The same request whole, in portions and token by token: equal within rounding of the compute type."""
+    folder = folders(name, stored_as(dtype))
+    toks = helpers.random_tokens(60, CONFIGS[name]["vocab"], 10)
+    a = helpers.replay_in_process(session_for(folder, dtype, 64), whole({"r": toks}))
+    trace = TraceBuilder().step([("r", toks[:31], "all")]).step([("r", toks[31:33], "all")])
+    for i in range(33, 60):
+        trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == 59 else [])
+    b = helpers.replay_in_process(session_for(folder, dtype, 64), trace)
+    if dtype == "float32":
+        assert max(helpers.worst(b[k], a[k]) for k in a) <= 1e-5
+    else:
+        assert max(helpers.worst(b[k], a[k]) / bound_at(folder, toks, k[1], dtype) for k in a) <= 2.0
+
+
+# --------------------------------------------------------------------------- batches, pages and slots used again
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_pages_and_slots_used_again(folders, name, dtype):
+    from tests.test_replay_gpu import mixed_trace
+    folder = folders(name, stored_as(dtype))
+    vocab = CONFIGS[name]["vocab"]
+    lengths = [33, 1, 90, 17, 64, 5, 48, 2, 71]
+    reqs = {f"q{i}": helpers.random_tokens(n, vocab, 40 + i) for i, n in enumerate(lengths)}
+    trace, peak = mixed_trace(reqs, max_live=3, seed=3)
+    session = session_for(folder, dtype, peak, max_requests=3)
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == sum(lengths)
+    check(got, folder, reqs, dtype, narrow=name == "B")
+    session.manager.check_invariants()
+    assert session.manager.slots.num_free == session.manager.slots.num_slots == 3
+    assert all(session.manager.num_free_pages(g) == session.manager.num_pages(g) for g in session.manager.groups)
+    kinds = {"prompt" if key[0] == "prompt" else "decode" for key in session.runner._graphs}
+    assert kinds == {"prompt", "decode"}, "steps of both kinds were replayed from graphs"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_slot_that_held_another_request_starts_from_zero(folders, dtype):
+    """One state slot, a page pool of one request: the second request gets the slot (the first one's projected rows in
+    it) and the pages the first one left full."""
+    folder = folders("A", stored_as(dtype))
+    reqs = {"first": helpers.random_tokens(50, MUTA_A["vocab"], 60), "second": helpers.random_tokens(44, MUTA_A["vocab"], 61)}
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        trace.step([(rid, toks[:20], "all")])
+        trace.step([(rid, toks[20:22], "all")])
+        for i in range(22, len(toks)):
+            trace.step([(rid, toks[i:i + 1], "all")], end=[rid] if i == len(toks) - 1 else [])
+    session = session_for(folder, dtype, 64, max_requests=1)
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+
+
+# --------------------------------------------------------------------------- where random weights would hide a fault
+def aim_queries(cfg, tensors, toks, key_pos, query_positions, free_tokens):
+    """Change the embeddings of ``free_tokens`` (one per query position, used nowhere else) and put them at
+    ``query_positions`` so that head 0's query there, on the dimensions that are not rotated, is the key that
+    position ``key_pos`` of ``toks`` gets, and zero on the rotated ones: with a large ``scale`` that one score towers
+    over all others wherever the key is visible.  One layer, no repeated range.  Returns the new tokens."""
+    layer = cfg["layers"][0]
+    m, kind, eps = layer["mixer"], layer["type"], float(cfg["norm"]["eps"])
+    d, r = int(m["dim"]), int(m["rot"]["dims"])
+    f64 = lambda n: tensors[n].to(torch.float64)
+    toks = list(toks)
+    first = kind == "attention"
+
+    def projected(names, tokens):
+        h = plain.root_mean_square_norm(f64("embed")[torch.as_tensor(tokens)], eps, f64("l0.norm1"))
+        out = []
+        for n in names:
+            u = h @ f64(f"l0.mix.{n}").T
+            if first:
+                u = plain.time_convolution(u + f64(f"l0.mix.{n}.b"), f64(f"l0.mix.{n}.conv"))
+            out.append(u)
+        return out
+
+    target = projected(["k"], toks[:key_pos + 1])[0][key_pos, :d].clone()          # key head 0, before rotation
+    target[:r] = 0.0
+    unit = 1.0 + f64("l0.norm1")
+    wq = f64("l0.mix.q")[:d]
+    for pos, token in sorted(zip(query_positions, free_tokens)):
+        toks[pos] = token
+        if not first:
+            # q = W h and only its direction counts: the smallest h with W_q0 h = target, and an embedding e = h / (1 + w),
+            # whose normed row has h's direction whatever its length
+            h = torch.linalg.lstsq(wq, target[:, None]).solution[:, 0]
+            tensors["embed"][token] = (h / unit).to(tensors["embed"].dtype)
+            continue
+        # q_pos = sum_j w_j (W h_(pos - taps + 1 + j) + b): the earlier rows are known, and the row the norm returns has a
+        # fixed length (e / rms(e) * (1 + w)).  So aim at a * target with a small enough that the smallest solution is
+        # shorter than that, and fill up to the length with a vector that W_q0 maps to zero.
+        taps_w, b = f64("l0.mix.q.conv")[:d], f64("l0.mix.q.b")[:d]
+        tensors["embed"][token] = 0                         # (a zero embedding's normed row is zero, its projected row the bias)
+        known = projected(["q"], toks[:pos + 1])[0][pos, :d] - taps_w[:, -1] * b
+        null = torch.linalg.svd(wq, full_matrices=True).Vh[d]                       # W_q0 null = 0
+        for a in (1.0, 0.5, 0.25, 0.125, 0.0625):
+            rhs = (a * target - known) / taps_w[:, -1] - b
+            h = torch.linalg.lstsq(wq, rhs[:, None]).solution[:, 0]
+            qa, qb, qc = ((null / unit) ** 2).mean(), 2.0 * (h * null / unit ** 2).mean(), ((h / unit) ** 2).mean() - 1.0
+            if qc < 0:
+                break
+        assert qc < 0, "no embedding of unit root mean square aims this query"
+        t = (-qb + torch.sqrt(qb * qb - 4.0 * qa * qc)) / (2.0 * qa)
+        tensors["embed"][token] = ((h + t * null) / unit).to(tensors["embed"].dtype)
+    return toks
+
+
+def _edge_case(tmp_path, kind, dtype, size, key_pos, seed):
+    """A one-layer model whose mask has ``size``, a key at ``key_pos`` and queries aimed at it on both sides of the
+    place where it leaves sight.  Returns (folder, tokens, last position that sees it, first that does not)."""
+    if kind == "attention_2":
+        mixer = _window(heads=2, kv_heads=1, dim=32, vdim=16, size=size, rot_dims=4, base=100.0, scale=0.6)
+        edge_in = key_pos + size - 1
+    else:
+        mixer = _blocks(heads=2, kv_heads=1, dim=32, vdim=16, conv=3, size=size, rot_dims=4, base=100.0, scale=0.6)
+        edge_in = (key_pos // size + 1) * size - 1
+    cfg = model(64, 120, [_layer(kind, mixer)], eps=1e-6, mult=1.0)
+    n = edge_in + 6
+    toks = [5 + t % 100 for t in helpers.random_tokens(n, 100, seed)]
+    toks[key_pos] = 4                                       # the key's token stands nowhere else
+    made = {}
+
+    def edit(tensors):
+        if kind == "attention":
+            for name in ("q", "k", "v"):                     # taps of ordinary size, the last one well away from zero
+                w = tensors[f"l0.mix.{name}.conv"].float()
+                w[:, -1] = 1.0 + w[:, -1]
+                tensors[f"l0.mix.{name}.conv"] = w.to(tensors[f"l0.mix.{name}.conv"].dtype)
+        made["toks"] = aim_queries(cfg, tensors, toks, key_pos, [edge_in - 1, edge_in, edge_in + 1, edge_in + 2], [0, 1, 2, 3])
+    folder = write_folder(tmp_path, cfg, seed=seed, stored=stored_as(dtype), edit=edit)
+    return folder, made["toks"], edge_in, edge_in + 1
+
+
+def _assert_edge_shows(folder, toks, edge_in, edge_out, dtype):
+    """The plain implementation with a mask one position larger or smaller differs far beyond the bound at the edge."""
+    want = plain_logits(folder, toks)
+    for off_by in (-1, 1):
+        other = plain.read_config(folder)
+        other["layers"][0]["mixer"]["mask"]["size"] += off_by
+        moved = plain.forward(other, plain.load_weights(folder), toks).numpy()
+        pos = edge_in if off_by < 0 else edge_out
+        assert helpers.worst(moved[pos], want[pos]) > 5 * bound_at(folder, toks, pos, dtype), "the aimed key does not show at the edge"
+    return want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind,size,key_pos", [("attention_2", 9, 20), ("attention_2", 130, 3), ("attention_2", 64, 63),
+                                               ("attention", 9, 20), ("attention", 150, 151), ("attention", 64, 64)])
+def test_edges_of_windows_and_blocks_in_prompts_and_in_decoding(tmp_path, kind, size, key_pos, dtype):
+    """One key that the queries near the edge score far above all others: the last position that sees it and the
+    first that does not are compared whole, with the edge among decoded tokens, with everything behind the key decoded
+    and with the edge at the start of a portion of two tokens.  Small masks, masks of more than two pages (the key far
+    back, over page borders) and masks of exactly one page with the key on the page's first or last place."""
+    folder, toks, edge_in, edge_out = _edge_case(tmp_path, kind, dtype, size, key_pos, seed=31)
+    want = _assert_edge_shows(folder, toks, edge_in, edge_out, dtype)
+    n = len(toks)
+    traces = {"whole": prompt_then_single("r", toks, n), "edge decoded": prompt_then_single("r", toks, edge_in - 3),
+              "all decoded": prompt_then_single("r", toks, key_pos + 1),
+              "edge starts a portion": TraceBuilder().step([("r", toks[:edge_in], "all")]).step([("r", toks[edge_in:edge_in + 2], "all")])
+              .step([("r", toks[edge_in + 2:], "all")], end=["r"])}
+    for label, trace in traces.items():
+        got = helpers.replay_in_process(session_for(folder, dtype, -(-n // 64) * 64), trace)
+        for pos in (edge_in - 1, edge_in, edge_out, edge_out + 1):
+            err = helpers.worst(got["r", pos], want[pos])
+            assert err <= 2.0 * bound_at(folder, toks, pos, dtype), f"{label}, position {pos}: {err:.3g}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_key_far_back_among_hundreds(tmp_path, dtype):
+    """A window of 400 positions, the aimed key 390 tokens back among as many others, over six page borders, through
+    portions and decoded tokens; without that key's token the plain logits differ far beyond the bound."""
+    folder, toks, edge_in, edge_out = _edge_case(tmp_path, "attention_2", dtype, 400, 7, seed=37)
+    want = _assert_edge_shows(folder, toks, edge_in, edge_out, dtype)
+    trace, at = TraceBuilder(), 0
+    for n in (17, 2, 64, 100, 3, 96, 60):
+        trace.step([("r", toks[at:at + n], "last")])
+        at += n
+    for i in range(at, len(toks)):
+        trace.step([("r", toks[i:i + 1], "all")], end=["r"] if i == len(toks) - 1 else [])
+    got = helpers.replay_in_process(session_for(folder, dtype, 448), trace)
+    check(got, folder, {"r": toks}, dtype)
+    assert ("r", edge_in) in got and ("r", edge_out) in got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_logits_without_a_key_in_the_softmax(tmp_path, dtype):
+    """Per-head logits of +3 and -2 in the denominator: the first tokens of every block, where few keys stand beside
+    them, lose most of their weight to the large ones.  Without them the plain logits differ far beyond the bound."""
+    cfg = ALONE["blocks"]
+
+    def edit(tensors):
+        tensors["l0.mix.sink"] = torch.tensor([3.0, -2.0, 2.5, 0.0]).to(tensors["l0.mix.sink"].dtype)
+    folder = write_folder(tmp_path, cfg, seed=41, stored=stored_as(dtype), edit=edit)
+    toks = helpers.random_tokens(40, cfg["vocab"], 15)
+    want = plain_logits(folder, toks)
+    weights = plain.load_weights(folder)
+    weights["l0.mix.sink"] = torch.full_like(weights["l0.mix.sink"], -1e4)
+    without = plain.forward(plain.read_config(folder), weights, toks).numpy()
+    assert min(helpers.worst(without[p], want[p]) for p in (0, 9, 18, 27)) > 5 * TOL["bfloat16"]
+    for cut in (40, 8, 1):
+        check(helpers.replay_in_process(session_for(folder, dtype, 64), prompt_then_single("r", toks, cut)), folder, {"r": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_experts_with_a_decisive_choice(tmp_path, dtype):
+    """Router rows made small and corrections set 0.05 apart in a shuffled order: the scores differ from token to token
+    by far less than that, so the choice (inside the two best of four groups) is the same under any rounding, while
+    the weights still differ from token to token.  Then bfloat16 rows of a model with experts can be held to the same
+    bounds as rows of a model without."""
+    cfg = ALONE["experts"]
+    order = [7, 2, 3, 0, 5, 1, 9, 10, 6, 11, 4, 8]           # groups 2 and 3 win; chosen: experts 6 and 7 and the first pass-through one
+
+    def edit(tensors):
+        tensors["l0.mlp.router"] = (tensors["l0.mlp.router"].float() * 0.05).to(tensors["l0.mlp.router"].dtype)
+        tensors["l0.mlp.correction"] = torch.tensor([0.05 * o for o in order]).to(tensors["l0.mlp.correction"].dtype)
+    folder = write_folder(tmp_path, cfg, seed=43, stored=stored_as(dtype), edit=edit)
+    toks = helpers.random_tokens(80, cfg["vocab"], 16)
+    chosen, weights = plain.route(plain.root_mean_square_norm(plain.load_weights(folder)["embed"].float()[toks], 1e-5),
+                                  plain.load_weights(folder)["l0.mlp.router"], plain.load_weights(folder)["l0.mlp.correction"], cfg["layers"][0]["mlp"]["router"])
+    assert {tuple(sorted(c)) for c in chosen.tolist()} == {(6, 7, 9)} and float(weights.std()) > 1e-4
+    got = helpers.replay_in_process(session_for(folder, dtype, 128), prompt_then_single("r", toks, 60))
+    want = plain_logits(folder, toks)
+    for (rid, pos), row in got.items():
+        err = helpers.worst(row, want[pos])
+        assert err <= 2.0 * bound_at(folder, toks, pos, dtype), (pos, err)
+
+
+def test_the_router_against_the_plain_choice():
+    """The routing kernel alone on rows made so that the choice is hard: corrections that are negative everywhere (a
+    group that is shut out must not win with a zero), groups whose best member is not among the best experts,
+    pass-through experts inside the last group, every expert chosen."""
+    from paged_llm_amd.csrc import ops
+    gen = torch.Generator().manual_seed(3)
+    for n, groups, keep, top, shift in [(12, 4, 2, 3, -2.0), (16, 4, 1, 4, 0.0), (18, 3, 2, 5, -0.5), (7, 7, 3, 3, 0.3), (8, 1, 1, 8, -1.0), (6, 2, 2, 1, 0.0)]:
+        h = torch.randn((64, 40), generator=gen)
+        w = torch.randn((n, 40), generator=gen) * 0.4
+        corr = torch.randn((n,), generator=gen) * 0.2 + shift
+        r = {"groups": {"count": groups, "keep": keep}, "top": top}
+        want_ids, want_w = plain.route(h, w, corr, r)
+        ids, weights = ops.moe_route(h.cuda(), w.cuda(), corr.cuda(), groups, keep, top)
+        ids, weights = ids.cpu().long(), weights.cpu()
+        order_a, order_b = ids.sort(dim=1), want_ids.sort(dim=1)
+        assert torch.equal(order_a.values, order_b.values), (n, groups, keep, top)
+        assert torch.allclose(torch.gather(weights, 1, order_a.indices), torch.gather(want_w, 1, order_b.indices), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    folder = folders("A", stored_as(dtype))
+    toks = helpers.random_tokens(300, MUTA_A["vocab"], 14)
+    trace = TraceBuilder().step([("r", toks[:4], "all")])
+    for i in range(4, 300):
+        trace.step([("r", toks[i:i + 1], "all" if i % 7 == 0 or i > 280 else [])], end=["r"] if i == 299 else [])
+    check(helpers.replay_in_process(session_for(folder, dtype, 320), trace), folder, {"r": toks}, dtype)
+
+
+# --------------------------------------------------------------------------- the entry point and its scheduler
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_greedy_generation_through_the_engine(folders, name):
+    """``LLMEngine.generate`` with portions of 16 tokens, three requests at a time for five prompts (state slots and
+    pages are used again): every row the engine sampled from is within the bound of the plain logits along its own
+    tokens, and in float32 the tokens are the plain implementation's greedy choice."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    vocab = CONFIGS[name]["vocab"]
+    prompts = [helpers.random_tokens(n, vocab, 70 + n) for n in (3, 41, 18, 1, 29)]
+    for dtype in ("float32", "bfloat16"):
+        folder = folders(name, stored_as(dtype))
+        engine = LLMEngine(folder, EngineConfig(dtype=dtype, num_gpu_blocks=24, block_size=16, max_num_batched_tokens=16,
+                                                max_num_seqs=3, max_model_len=128))
+        rows = {}
+
+        def keep(requests, logits):
+            for r, row in zip(requests, logits.float().cpu()):
+                rows[r.id, len(r.tokens) - 1] = row.numpy()
+        engine.on_logits = keep
+        outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+        assert engine.cache_manager.slots.num_free == 3
+        for p, o in zip(prompts, outs):
+            assert len(o.token_ids) == 12
+            want = plain_logits(folder, p + o.token_ids)
+            for i, token in enumerate(o.token_ids):
+                pos = len(p) + i - 1
+                err = helpers.worst(rows[o.seq_id, pos], want[pos])
+                assert err <= 2.0 * bound_at(folder, p + o.token_ids, pos, dtype) and int(rows[o.seq_id, pos].argmax()) == token, (dtype, pos, err)
+                if dtype == "float32":
+                    top2 = np.sort(want[pos])[-2:]
+                    if top2[1] - top2[0] > 1e-3 * np.abs(want[pos]).max():
+                        assert token == int(want[pos].argmax()), (pos, token)
+
+
+def test_the_command_line_generates(folders, capsys):
+    import importlib.util
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("generate_example", os.path.join(root, "examples", "generate.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    code = mod.main(["--model", folders("A", "bfloat16"), "--prompt-ids", "5,6,7", "--prompt-ids", "9", "--max-tokens", "6",
+                     "--num-gpu-blocks", "16", "--max-model-len", "64", "--ignore-eos"])
+    out = capsys.readouterr().out
+    assert code == 0 and "decode_tokens=" in out and out.count("--- [") == 2
+
+
+def test_the_replay_program(folders, tmp_path):
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = folders("A", "float32")
+    toks = {"a": helpers.random_tokens(70, MUTA_A["vocab"], 90), "b": helpers.random_tokens(45, MUTA_A["vocab"], 91)}
+    trace = TraceBuilder()
+    trace.step([("a", toks["a"][:50], [0, 49])])
+    trace.step([("a", toks["a"][50:52], "all"), ("b", toks["b"][:30], [])])
+    trace.step([("b", toks["b"][30:], "last"), ("a", toks["a"][52:53], "all")], end=["b"])
+    trace.step([("a", toks["a"][53:], "all")], end=["a"])
+    out_dir = tmp_path / "out"
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(out_dir),
+                           "--max-tokens", "192"], input=trace.jsonl(), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
+    got = helpers.read_replay_output(str(out_dir), trace, MUTA_A["vocab"])
+    assert len(got) == 2 + 2 + 1 + 1 + 17
+    check(got, folder, toks, "float32")
+
+
+# --------------------------------------------------------------------------- sizes drawn at random
+def random_configuration(seed: int) -> dict:
+    """A Mutapel configuration with every size drawn at random (small ones, ones and odd ones included), the two mixers
+    in a random order, some layers without a feed-forward, a repeated range or none."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *values: values[int(rng.integers(len(values)))]
+
+    def mixer(kind):
+        kv = pick(1, 2, 3)
+        heads = kv * pick(1, 2, 4)
+        dim = pick(2, 6, 16, 24, 34, 70)
+        rot = pick(*[r for r in (0, 2, 4, 6, 16, 34) if r <= dim])
+        common = dict(heads=heads, kv_heads=kv, dim=dim, vdim=pick(1, 3, 16, 40, 66), size=pick(1, 2, 7, 16, 33, 64, 100),
+                      rot_dims=rot, base=pick(10.0, 1e4, 1e6), scale=float(rng.uniform(0.05, 0.5)))
+        return _blocks(conv=pick(1, 2, 4, 5), **common) if kind == "attention" else _window(**common)
+
+    def mlp():
+        if rng.random() < 0.25:
+            return None
+        count = pick(1, 2, 3, 4)
+        per = pick(1, 2, 3)
+        n = count * per
+        identity = pick(*[i for i in (0, 1, 2, n - 1) if 0 <= i < n])
+        keep = pick(*range(1, count + 1))
+        return _moe(experts=n - identity, identity=identity, top=pick(*range(1, per * keep + 1)), count=count, keep=keep, ff=pick(8, 10, 36, 65))
+
+    n = int(rng.integers(1, 5))
+    layers = []
+    for _ in range(n):
+        kind = pick("attention", "attention_2")
+        layers.append(_layer(kind, mixer(kind), mlp()))
+    loop = None
+    if rng.random() < 0.7:
+        start = int(rng.integers(0, n))
+        loop = (start, int(rng.integers(start + 1, n + 1)), pick(1, 2, 3))
+    return model(pick(16, 30, 48, 66, 100), pick(40, 97, 300), layers, loop=loop, eps=pick(1e-6, 1e-5, 1e-3), mult=float(rng.uniform(0.2, 1.2)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    """Whatever the sizes, the engine computes what the plain implementation computes, whole, in portions and token by
+    token, two requests side by side."""
+    cfg = random_configuration(seed)
+    folder = write_folder(tmp_path, cfg, seed=100 + seed, stored=stored_as(dtype))
+    reqs = {"a": helpers.random_tokens(150, cfg["vocab"], 200 + seed), "b": helpers.random_tokens(37, cfg["vocab"], 300 + seed)}
+    trace = TraceBuilder()
+    trace.step([("a", reqs["a"][:130], "all")])
+    trace.step([("a", reqs["a"][130:132], "all"), ("b", reqs["b"][:20], "all")])
+    for i in range(17):
+        trace.step([("a", reqs["a"][132 + i:133 + i], "all"), ("b", reqs["b"][20 + i:21 + i], "all")], end=["b"] if i == 16 else [])
+    trace.step([("a", reqs["a"][149:], "all")], end=["a"])
+    got = helpers.replay_in_process(session_for(folder, dtype, 256), trace)
+    assert len(got) == 150 + 37
+    check(got, folder, reqs, dtype, narrow=True)
+
+
+def test_preempted_requests_are_computed_again_from_their_first_token(tmp_path):
+    """A page pool too small for three requests at once: the scheduler preempts the request admitted last (pages and
+    state slot given back, its tokens kept) and computes it again later as a longer prompt.  Float32: the tokens are
+    the plain implementation's greedy choice all the same."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    cfg = copy.deepcopy(MUTA_A)
+    for layer in cfg["layers"]:
+        layer["mixer"]["mask"]["size"] = 200                # nothing leaves sight, so no page goes back while a request runs
+    folder = write_folder(tmp_path, cfg, seed=29, stored="float32")
+    vocab = cfg["vocab"]
+    prompts = [helpers.random_tokens(n, vocab, 400 + n) for n in (30, 22, 27)]
+    engine = LLMEngine(folder, EngineConfig(dtype="float32", num_gpu_blocks=10, block_size=16, max_num_batched_tokens=32,
+                                            max_num_seqs=3, max_model_len=128))
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True))
+    assert engine.stats.num_preemptions > 0 and sum(o.num_preemptions for o in outs) > 0
+    assert engine.cache_manager.slots.num_free == 3
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 40
+        want = plain_logits(folder, p + o.token_ids)
+        for i, token in enumerate(o.token_ids):
+            row = want[len(p) + i - 1]
+            top2 = np.sort(row)[-2:]
+            if top2[1] - top2[0] > 1e-3 * np.abs(row).max():
+                assert token == int(row.argmax()), (len(p), i)
