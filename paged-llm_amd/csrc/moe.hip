@@ -6,7 +6,8 @@
 //   moe_align      the (token, choice) pairs sorted by expert: per expert a run of rows, cut into tiles of rows;
 //   moe_expert_gemm the experts' products over those runs: act(gate h) * (up h) from the tokens' rows, and the down
 //                  product from the activations; one tile of rows per workgroup, every row's sums in ascending k,
-//                  so a pair's result does not depend on which other pairs share its tile or in which order;
+//                  so a pair's result does not depend on which other pairs share its tile or in which order
+//                  (bfloat16: on the matrix cores; float32, and sizes that fit no 16-byte load: plain multiply-adds);
 //   moe_combine    out[t] = sum over the token's choices, in their order, of weight * (expert output | the token's row).
 //
 // Router, softmax, weights and the final sum are float; T is the storage type of rows, activations and matrices.
@@ -14,7 +15,8 @@
 
 using namespace pllm;
 
-constexpr int kMoeTileRows = 16;   // rows (pairs) of one tile of the experts' products
+constexpr int kMoeTileRows = 16;      // rows (pairs) of the smallest tile of the experts' products
+constexpr int kMoeMaxTileRows = 64;   // ... and of the largest (steps with many pairs per expert)
 
 // ---------------------------------------------------------------------------------------------
 // n = experts + pass-through experts router outputs; groups of n / groups neighbours; a group's mark is its largest
@@ -30,12 +32,31 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = h + (size_t)t * ld;
-  for (int e = wave; e < n; e += 4) {
-    const float* w = router_w + (size_t)e * width;
-    float acc = 0.f;
-    for (int i = lane; i < width; i += 64) acc = fmaf(to_f32(row[i]), w[i], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) score[e] = acc;
+  // a wavefront takes eight router rows at a time: one pass over the token's row with eight independent loads and sums
+  // per element (one row at a time is a chain of dependent loads: 100 us for 32 rows of 2,048)
+  for (int e0 = wave * 8; e0 < n; e0 += 32) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const float* w = router_w + (size_t)e0 * width;
+    if (e0 + 8 <= n) {
+#pragma unroll 4
+      for (int i = lane; i < width; i += 64) {
+        const float x = to_f32(row[i]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = fmaf(x, w[(size_t)j * width + i], acc[j]);
+      }
+    } else {
+      for (int i = lane; i < width; i += 64) {
+        const float x = to_f32(row[i]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (e0 + j < n) acc[j] = fmaf(x, w[(size_t)j * width + i], acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float total = wave_sum(acc[j]);
+      if (lane == 0 && e0 + j < n) score[e0 + j] = total;
+    }
   }
   __syncthreads();
   if (threadIdx.x != 0) return;
@@ -96,12 +117,12 @@ PLLM_API int pllm_moe_route(int dtype, const void* h, int ld, const float* route
 // ids [pairs] -> the pairs of experts < `experts` sorted by expert.
 //   sorted_pair [pairs]   the pair at each sorted row (rows past the last one: untouched)
 //   row_of_pair [pairs]   the sorted row of each pair, -1 for a pass-through expert
-//   tiles [max_tiles][3]  (expert, first row, rows) of every tile of at most kMoeTileRows rows; tiles[.][2] = 0 past the last
+//   tiles [max_tiles][3]  (expert, first row, rows) of every tile of at most tile_rows rows; tiles[.][2] = 0 past the last
 // One workgroup; the order of the pairs of one expert is whatever the atomics give (the products do not depend on it).
 constexpr int kMoeMaxExperts = 1024;
 
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int pairs, int experts, int* __restrict__ sorted_pair,
-                                                         int* __restrict__ row_of_pair, int* __restrict__ tiles, int max_tiles) {
+                                                         int* __restrict__ row_of_pair, int* __restrict__ tiles, int max_tiles, int tile_rows) {
   __shared__ int count[kMoeMaxExperts], first[kMoeMaxExperts], cursor[kMoeMaxExperts];
   for (int e = threadIdx.x; e < experts; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
   __syncthreads();
@@ -114,10 +135,10 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
     int at = 0, nt = 0;
     for (int e = 0; e < experts; ++e) {
       first[e] = at;
-      for (int r = 0; r < count[e] && nt < max_tiles; r += kMoeTileRows, ++nt) {
+      for (int r = 0; r < count[e] && nt < max_tiles; r += tile_rows, ++nt) {
         tiles[3 * nt] = e;
         tiles[3 * nt + 1] = at + r;
-        tiles[3 * nt + 2] = min(kMoeTileRows, count[e] - r);
+        tiles[3 * nt + 2] = min(tile_rows, count[e] - r);
       }
       at += count[e];
     }
@@ -137,10 +158,11 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
 }
 
 PLLM_API int pllm_moe_align(const int* ids, int pairs, int experts, int* sorted_pair, int* row_of_pair, int* tiles, int max_tiles,
-                            hipStream_t stream) {
+                            int tile_rows, hipStream_t stream) {
   if (pairs <= 0) return 0;
-  if (experts <= 0 || experts > kMoeMaxExperts || max_tiles < (pairs + kMoeTileRows - 1) / kMoeTileRows + experts) return -2;
-  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, sorted_pair, row_of_pair, tiles, max_tiles);
+  if (tile_rows < kMoeTileRows || tile_rows % kMoeTileRows || tile_rows > kMoeMaxTileRows) return -2;
+  if (experts <= 0 || experts > kMoeMaxExperts || max_tiles < (pairs + tile_rows - 1) / tile_rows + experts) return -2;
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, sorted_pair, row_of_pair, tiles, max_tiles, tile_rows);
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -200,10 +222,144 @@ __global__ __launch_bounds__(256) void moe_expert_gemm_kernel(const T* __restric
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same products in bfloat16 on the matrix cores (v_mfma_f32_16x16x32_bf16), operands straight from memory into the
+// registers the instruction reads: lane (r, g) = (lane & 15, lane >> 4) holds elements 8 g .. 8 g + 7 of row r of a
+// k-step of 32, for the tile's rows (gathered through sorted_pair for the gated product) and for 16 weight rows alike.
+// A workgroup is one tile of MT * 16 rows of one expert times 4 wavefronts * U blocks of 16 outputs (gated: the
+// gate's and the up product's 16 rows each); a wavefront keeps U * MT (gated: 2 U MT) accumulators.  In steps of few
+// tokens (MT = 1) every wavefront streams weight rows that no other one reads, which is all there is to do: such a step
+// is bound by the chosen experts' bytes.  In prompt steps (tiles of 64 rows) the four wavefronts read the same rows
+// (the first one's misses are the others' cache hits) and each of its own weight rows once per 64 rows.
+// An output element is one accumulator over ascending k-steps whatever MT and U are, so its value does not depend on
+// the tile it is in, the kernel's shape or the other rows.  K % 8 == 0, ld_in % 8 == 0; a last k-step beyond K reads zeros.
+typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float moe_floatx4;
+
+template <bool GATED, int MT, int U>
+__global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __restrict__ rows_in, int ld_in, const bf16* __restrict__ w,
+                                                              const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
+                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act) {
+  constexpr int W = GATED ? 2 : 1;
+  const int tile = blockIdx.x;
+  const int expert = tiles[3 * tile], row0 = tiles[3 * tile + 1], nrows = tiles[3 * tile + 2];
+  if (nrows <= 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int block0 = (blockIdx.y * 4 + wave) * U;           // this wavefront's first block of 16 outputs
+  if (block0 * 16 >= n_out) return;
+  const bf16* a_ptr[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int row = row0 + min(t * 16 + r, nrows - 1);       // rows past the tile's last repeat it: never stored
+    const int src = GATED ? sorted_pair[row] / top : row;
+    a_ptr[t] = rows_in + (size_t)src * ld_in + 8 * g;
+  }
+  const bf16* we = w + (size_t)expert * W * n_out * K;
+  const bf16* w_ptr[U][W];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int col = min((block0 + u) * 16 + r, n_out - 1);   // outputs past the last repeat it: never stored
+#pragma unroll
+    for (int h = 0; h < W; ++h) w_ptr[u][h] = we + ((size_t)h * n_out + col) * K + 8 * g;
+  }
+  moe_floatx4 acc[U][W][MT];
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int h = 0; h < W; ++h)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[u][h][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  const int k_whole = K & ~31;
+#pragma unroll 2
+  for (int k0 = 0; k0 < k_whole; k0 += 32) {
+    moe_bf16x8 a[MT], b[U][W];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) a[t] = *reinterpret_cast<const moe_bf16x8*>(a_ptr[t] + k0);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int h = 0; h < W; ++h) b[u][h] = *reinterpret_cast<const moe_bf16x8*>(w_ptr[u][h] + k0);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int h = 0; h < W; ++h)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[u][h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][h], a[t], acc[u][h][t], 0, 0, 0);
+  }
+  if (k_whole < K) {                                         // the last, partial k-step: lanes whose eight elements lie beyond K hold zeros
+    const bool in = k_whole + 8 * g < K;
+    const moe_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    moe_bf16x8 a[MT], b[U][W];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) a[t] = in ? *reinterpret_cast<const moe_bf16x8*>(a_ptr[t] + k_whole) : zero;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int h = 0; h < W; ++h) b[u][h] = in ? *reinterpret_cast<const moe_bf16x8*>(w_ptr[u][h] + k_whole) : zero;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int h = 0; h < W; ++h)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[u][h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][h], a[t], acc[u][h][t], 0, 0, 0);
+  }
+  // a lane's four sums: outputs 4 g .. 4 g + 3 of its block, for row r of every row tile
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int row = t * 16 + r;
+    if (row >= nrows) continue;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int col = (block0 + u) * 16 + 4 * g;
+      if (col >= n_out) continue;
+      if (GATED) {
+        bf16* o = reinterpret_cast<bf16*>(out_) + (size_t)(row0 + row) * ld_out + col;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[u][0][t][i], act) * acc[u][W - 1][t][i]);
+      } else {
+        float* o = reinterpret_cast<float*>(out_) + (size_t)(row0 + row) * ld_out + col;
+        if (col + 3 < n_out && (ld_out & 3) == 0) {
+          *reinterpret_cast<float4*>(o) = make_float4(acc[u][0][t][0], acc[u][0][t][1], acc[u][0][t][2], acc[u][0][t][3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (col + i < n_out) o[i] = acc[u][0][t][i];
+        }
+      }
+    }
+  }
+}
+
+template <bool GATED>
+static void launch_moe_mfma(int tile_rows, int max_tiles, const bf16* rows_in, int ld_in, const bf16* w, const int* tiles,
+                            const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, hipStream_t stream) {
+  const int blocks = (n_out + 15) / 16;
+  if (tile_rows >= 64) {
+    constexpr int U = GATED ? 1 : 2;
+    dim3 grid(max_tiles, (blocks + 4 * U - 1) / (4 * U));
+    hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 4, U>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
+  } else {
+    dim3 grid(max_tiles, (blocks + 3) / 4);
+    hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 1, 1>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
+  }
+}
+
+// tile_rows: what moe_align was given.  Tiles of more than 16 rows are for the matrix-core kernel alone (bfloat16,
+// K and ld_in multiples of 8, 16-byte aligned operands); the plain kernel takes tiles of 16.
 PLLM_API int pllm_moe_expert_gemm(int dtype, int gated, const void* rows_in, int ld_in, const void* w, const int* tiles, int max_tiles,
-                                  const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, hipStream_t stream) {
+                                  int tile_rows, const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act,
+                                  hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || K <= 0 || top <= 0 || act < 0 || act >= PLLM_ACT_COUNT) return -2;
+  const bool matrix_cores = dtype == PLLM_BF16 && K % 8 == 0 && ld_in % 8 == 0 && ((uintptr_t)rows_in & 15) == 0 && ((uintptr_t)w & 15) == 0;
+  if (tile_rows != kMoeTileRows && !(matrix_cores && tile_rows == kMoeMaxTileRows)) return -2;
+  if (matrix_cores) {
+    if (gated) launch_moe_mfma<true>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, stream);
+    else launch_moe_mfma<false>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, stream);
+    PLLM_RETURN_LAST_ERROR();
+  }
   dim3 grid(max_tiles, (n_out + kMoeCols - 1) / kMoeCols), block(256);
 #define PLLM_MOE(T, G)                                                                                                         \
   hipLaunchKernelGGL((moe_expert_gemm_kernel<T, G>), grid, block, 0, stream, (const T*)rows_in, ld_in, (const T*)w, tiles,    \

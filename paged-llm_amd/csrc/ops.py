@@ -1487,6 +1487,7 @@ def gate_heads(o: torch.Tensor, gate: torch.Tensor | None, heads: int, dv: int, 
 
 # ------------------------------------------------------------------------------------------- routed experts
 MOE_TILE_ROWS = 16
+MOE_MAX_TILE_ROWS = 64
 MOE_MAX_EXPERTS = 1024
 
 
@@ -1511,25 +1512,35 @@ def moe_route(h: torch.Tensor, router_w: torch.Tensor, correction: torch.Tensor 
     return ids, weights
 
 
-def moe_align(ids: torch.Tensor, experts: int) -> tuple:
+def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, *inner_sizes: int) -> int:
+    """Rows of a tile of the experts' products for a step of ``pairs`` (token, choice) pairs: 64 where the matrix-core
+    kernel runs (bfloat16, every product's inner size a multiple of 8) and an expert gets 32 pairs or more on average,
+    else 16.  It depends on the step's number of tokens only, so a replayed step keeps its choice."""
+    if dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes) and pairs >= 32 * experts:
+        return MOE_MAX_TILE_ROWS
+    return MOE_TILE_ROWS
+
+
+def moe_align(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> tuple:
     """The (token, choice) pairs of ``ids`` [T, top] whose expert is below ``experts``, sorted by expert:
     (sorted_pair int32 [pairs], row_of_pair int32 [pairs] (-1: an expert without weights), tiles int32 [max_tiles, 3]
-    of (expert, first row, rows), rows 0 past the last tile)."""
+    of (expert, first row, rows) with at most ``tile_rows`` rows each, rows 0 past the last tile)."""
     _on_gpu(ids)
     _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "ids: contiguous int32 [T, top]")
     _need(0 < experts <= MOE_MAX_EXPERTS, f"1 to {MOE_MAX_EXPERTS} experts")
+    _need(tile_rows in (MOE_TILE_ROWS, MOE_MAX_TILE_ROWS), f"tiles of {MOE_TILE_ROWS} or {MOE_MAX_TILE_ROWS} rows")
     pairs = ids.numel()
-    max_tiles = -(-pairs // MOE_TILE_ROWS) + experts
+    max_tiles = -(-pairs // tile_rows) + experts
     sorted_pair = torch.empty(pairs, dtype=torch.int32, device=ids.device)
     row_of_pair = torch.empty(pairs, dtype=torch.int32, device=ids.device)
     tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=ids.device)
-    _check(_fn("moe.hip", "pllm_moe_align", signature=[c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p])(
-        _ptr(ids), pairs, experts, _ptr(sorted_pair), _ptr(row_of_pair), _ptr(tiles), max_tiles, _stream()), "moe_align")
+    _check(_fn("moe.hip", "pllm_moe_align", signature=[c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p])(
+        _ptr(ids), pairs, experts, _ptr(sorted_pair), _ptr(row_of_pair), _ptr(tiles), max_tiles, tile_rows, _stream()), "moe_align")
     return sorted_pair, row_of_pair, tiles
 
 
 def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor, sorted_pair: torch.Tensor, top: int, gated: bool,
-                    activation: str = "silu") -> torch.Tensor:
+                    activation: str = "silu", tile_rows: int = MOE_TILE_ROWS) -> torch.Tensor:
     """The experts' products over the sorted pairs.  ``gated``: rows_in [T, K] are the tokens' rows, w [experts, 2 N, K]
     holds [gate; up] per expert, the result [pairs, N] in the rows' type is act(gate . a) * (up . a) for the pair's token.
     Else rows_in [pairs, K] are rows in sorted order, w [experts, N, K], and the result is float32 [pairs, N]."""
@@ -1538,15 +1549,17 @@ def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor,
           and w.shape[2] == rows_in.shape[1], f"moe_expert_gemm shapes {tuple(rows_in.shape)} x {tuple(w.shape)}")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous(), "tiles: int32 [n, 3]")
     pairs = sorted_pair.numel()
-    _need(sorted_pair.dtype == torch.int32 and sorted_pair.is_contiguous() and tiles.shape[0] >= -(-pairs // MOE_TILE_ROWS), "sorted pairs and their tiles")
+    _need(sorted_pair.dtype == torch.int32 and sorted_pair.is_contiguous() and tiles.shape[0] >= -(-pairs // tile_rows), "sorted pairs and their tiles")
+    _need(tile_rows == MOE_TILE_ROWS or (tile_rows == MOE_MAX_TILE_ROWS and rows_in.dtype == torch.bfloat16 and rows_in.shape[1] % 8 == 0
+                                         and rows_in.stride(0) % 8 == 0), "tiles of 64 rows are the matrix-core kernel's")
     K = rows_in.shape[1]
     N = w.shape[1] // 2 if gated else w.shape[1]
     _need(gated or rows_in.shape[0] == pairs, "the down product takes one row per pair")
     _need(not gated or (w.shape[1] % 2 == 0 and rows_in.shape[0] * top == pairs), "the gated product takes the tokens' rows")
     out = torch.empty((pairs, N), dtype=rows_in.dtype if gated else torch.float32, device=rows_in.device)
-    _check(_fn("moe.hip", "pllm_moe_expert_gemm", signature=[c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+    _check(_fn("moe.hip", "pllm_moe_expert_gemm", signature=[c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
                                                               c_void_p, c_int, c_int, c_void_p])(
-        dtype_code(rows_in.dtype), int(gated), _ptr(rows_in), rows_in.stride(0), _ptr(w), _ptr(tiles), tiles.shape[0], _ptr(sorted_pair), top, N, K,
+        dtype_code(rows_in.dtype), int(gated), _ptr(rows_in), rows_in.stride(0), _ptr(w), _ptr(tiles), tiles.shape[0], tile_rows, _ptr(sorted_pair), top, N, K,
         _ptr(out), out.stride(0), activation_code(activation), _stream()), "moe_expert_gemm")
     return out
 

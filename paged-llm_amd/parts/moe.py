@@ -75,9 +75,10 @@ class RoutedExperts(FeedForward):
     def forward(self, h, ctx):
         h = rows_of(h)
         ids, weights = ops.moe_route(h, self.router, self.correction, self.groups, self.keep, self.top)
-        sorted_pair, row_of_pair, tiles = ops.moe_align(ids, self.experts)
-        act = ops.moe_expert_gemm(h, self.w_gate_up, tiles, sorted_pair, self.top, True, self.activation)
-        out = ops.moe_expert_gemm(act, self.w_down, tiles, sorted_pair, self.top, False)
+        rows = ops.moe_tile_rows(ids.numel(), self.experts, h.dtype, self.hidden, self.inter, h.stride(0))
+        sorted_pair, row_of_pair, tiles = ops.moe_align(ids, self.experts, rows)
+        act = ops.moe_expert_gemm(h, self.w_gate_up, tiles, sorted_pair, self.top, True, self.activation, tile_rows=rows)
+        out = ops.moe_expert_gemm(act, self.w_down, tiles, sorted_pair, self.top, False, tile_rows=rows)
         y = ops.moe_combine(out, h, row_of_pair, weights)
         if getattr(ctx, "float_branch", False):
             return y

@@ -449,6 +449,41 @@ def test_the_router_against_the_plain_choice():
         assert torch.allclose(torch.gather(weights, 1, order_a.indices), torch.gather(want_w, 1, order_b.indices), rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("tokens,width,ff,experts,top", [(5, 64, 32, 3, 2), (200, 96, 40, 4, 3), (300, 128, 72, 2, 1), (131, 40, 100, 5, 5)])
+def test_the_experts_products_on_the_matrix_cores(tokens, width, ff, experts, top):
+    """The bfloat16 kernels of the experts' products (tiles of 16 and of 64 rows; inner sizes with a partial last step
+    of 32; outputs that fill no block of 16) against float64 sums over the same bfloat16 operands, and a pair's row
+    bit for bit the same whatever the tile size."""
+    from paged_llm_amd.csrc import ops
+    gen = torch.Generator().manual_seed(tokens)
+    h = torch.randn((tokens, width), generator=gen).to(torch.bfloat16).cuda()
+    w1 = (torch.randn((experts, 2 * ff, width), generator=gen) * width ** -0.5).to(torch.bfloat16).cuda()
+    w2 = (torch.randn((experts, width, ff), generator=gen) * ff ** -0.5).to(torch.bfloat16).cuda()
+    ids = torch.stack([torch.randperm(experts + 1, generator=gen)[:top] for _ in range(tokens)]).to(torch.int32).cuda()   # (expert `experts`: a pass-through one)
+    results = []
+    for rows in (ops.MOE_TILE_ROWS, ops.MOE_MAX_TILE_ROWS):
+        if rows != ops.MOE_TILE_ROWS and (width % 8 or ff % 8):
+            continue                                        # (the plain kernel takes over; it has tiles of 16 rows only)
+        sorted_pair, row_of_pair, tiles = ops.moe_align(ids, experts, rows)
+        act = ops.moe_expert_gemm(h, w1, tiles, sorted_pair, top, True, "silu", tile_rows=rows)
+        out = ops.moe_expert_gemm(act, w2, tiles, sorted_pair, top, False, tile_rows=rows)
+        torch.cuda.synchronize()
+        place = row_of_pair.cpu().long()
+        keep = place >= 0
+        assert int(keep.sum()) == int((ids < experts).sum()) and sorted(place[keep].tolist()) == list(range(int(keep.sum())))
+        results.append((act.cpu()[place[keep]], out.cpu()[place[keep]]))
+        pair = torch.nonzero(keep)[:, 0]
+        token, expert = pair // top, ids.cpu().long().flatten()[pair]
+        x = h.cpu().double()[token]
+        gu = torch.einsum("pk,pnk->pn", x, w1.cpu().double()[expert])
+        want_act = torch.nn.functional.silu(gu[:, :ff]) * gu[:, ff:]
+        assert torch.allclose(results[-1][0].double(), want_act, rtol=2e-2, atol=2e-2 * float(want_act.abs().max()))
+        want_out = torch.einsum("pk,pnk->pn", results[-1][0].double(), w2.cpu().double()[expert])
+        assert torch.allclose(results[-1][1].double(), want_out, rtol=1e-4, atol=1e-5 * float(want_out.abs().max()))
+    if len(results) == 2:
+        assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     folder = folders("A", stored_as(dtype))
