@@ -16,36 +16,46 @@
 using namespace pllm;
 
 constexpr int kMoeTileRows = 16;      // rows (pairs) of the smallest tile of the experts' products
-constexpr int kMoeMaxTileRows = 64;   // ... and of the largest (steps with many pairs per expert)
+constexpr int kMoeMaxTileRows = 128;  // ... and of the largest (steps with many pairs per expert); 64 in between
 
 // ---------------------------------------------------------------------------------------------
 // n = experts + pass-through experts router outputs; groups of n / groups neighbours; a group's mark is its largest
 // corrected score; only experts of the `keep` best groups can be chosen (ties: the lower index wins).
+constexpr int kRouteThreads = 1024, kRoutePieces = 16;   // threads of a workgroup in steps of few tokens; pieces the products are cut into
+
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ router_w,
-                                                        const float* __restrict__ correction, int width, int n, int groups, int keep,
-                                                        int top, int* __restrict__ ids, float* __restrict__ weights) {
+__global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ router_w,
+                                                                  const float* __restrict__ correction, int width, int n, int groups, int keep,
+                                                                  int top, int segments, int* __restrict__ ids, float* __restrict__ weights) {
   extern __shared__ float lds[];
   float* score = lds;            // [n]  router outputs, then scores
   float* choice = lds + n;       // [n]  score + correction, -inf once taken or shut out
   float* mark = lds + 2 * n;     // [groups]
+  float* part = mark + groups;   // [segments][n]  sums over a segment of the row
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = h + (size_t)t * ld;
-  // a wavefront takes eight router rows at a time: one pass over the token's row with eight independent loads and sums
-  // per element (one row at a time is a chain of dependent loads: 100 us for 32 rows of 2,048)
-  for (int e0 = wave * 8; e0 < n; e0 += 32) {
+  // The router's products.  A piece of work is eight router rows times one of `segments` equal parts of the token's
+  // row, and the wavefronts (16 in steps of few tokens, 4 in others) take the pieces in turn: one pass over the part with eight independent loads and sums
+  // per element, several elements under way (few tokens, a router matrix that the experts' weights have pushed out of
+  // the caches since the last layer: what counts is how few loads wait for one another).  A router output is the sum
+  // of its parts in ascending order, each part summed lane by lane and then over the wavefront.
+  const int batches = (n + 7) / 8;
+  const int seg = ((width + segments - 1) / segments + 63) & ~63;
+  for (int piece = wave; piece < batches * segments; piece += (int)(blockDim.x >> 6)) {
+    const int e0 = (piece / segments) * 8, sg = piece % segments;
+    const int from = sg * seg, to = min(width, from + seg);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const float* w = router_w + (size_t)e0 * width;
     if (e0 + 8 <= n) {
-#pragma unroll 4
-      for (int i = lane; i < width; i += 64) {
+#pragma unroll 8
+      for (int i = from + lane; i < to; i += 64) {
         const float x = to_f32(row[i]);
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j] = fmaf(x, w[(size_t)j * width + i], acc[j]);
       }
     } else {
-      for (int i = lane; i < width; i += 64) {
+      for (int i = from + lane; i < to; i += 64) {
         const float x = to_f32(row[i]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
@@ -55,47 +65,76 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float total = wave_sum(acc[j]);
-      if (lane == 0 && e0 + j < n) score[e0 + j] = total;
+      if (lane == 0 && e0 + j < n) part[sg * n + e0 + j] = total;
     }
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
-  float m = -INFINITY;
-  for (int e = 0; e < n; ++e) m = fmaxf(m, score[e]);
-  float sum = 0.f;
-  for (int e = 0; e < n; ++e) { score[e] = expf(score[e] - m); sum += score[e]; }
-  const float inv = 1.f / sum;
-  for (int e = 0; e < n; ++e) {
-    score[e] *= inv;
-    choice[e] = score[e] + (correction ? correction[e] : 0.f);
+  for (int e = threadIdx.x; e < n; e += blockDim.x) {
+    float total = part[e];
+    for (int sg = 1; sg < segments; ++sg) total += part[sg * n + e];
+    score[e] = total;
   }
+  __syncthreads();
+  // The choice, by the first wavefront (the others keep it company at the barriers): lane l looks after router outputs
+  // l, l + 64, ...; a largest element is found by a maximum over the wavefront and then the lowest index that holds it
+  // (ties: the lower index wins).
+  const bool chooser = wave == 0;
+  auto lowest_at = [&](const float* values, int count) {
+    float mine = -INFINITY;
+    for (int e = lane; e < count; e += 64) mine = fmaxf(mine, values[e]);
+    const float best = wave_max(mine);
+    float at = 3.0e9f;
+    for (int e = lane; e < count; e += 64)
+      if (values[e] == best) { at = (float)e; break; }
+    return (int)(-wave_max(-at));
+  };
+  if (chooser) {
+    float m = -INFINITY;
+    for (int e = lane; e < n; e += 64) m = fmaxf(m, score[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < n; e += 64) { const float x = expf(score[e] - m); score[e] = x; sum += x; }
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+    for (int e = lane; e < n; e += 64) {
+      const float sc = score[e] * inv;
+      score[e] = sc;
+      choice[e] = sc + (correction ? correction[e] : 0.f);
+    }
+  }
+  __syncthreads();
   const int per = n / groups;
   if (keep < groups) {
-    for (int g = 0; g < groups; ++g) {
-      float best = -INFINITY;
-      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, choice[e]);
-      mark[g] = best;
-    }
-    // the `keep` best groups get +inf as their mark; the others' experts are shut out
+    if (chooser)
+      for (int g = lane; g < groups; g += 64) {
+        float best = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, choice[e]);
+        mark[g] = best;
+      }
+    __syncthreads();
+    // the `keep` best groups are taken one by one (a taken group's mark becomes -inf); the others' experts are shut out
     for (int k = 0; k < keep; ++k) {
-      int at = -1;
-      float best = -INFINITY;
-      for (int g = 0; g < groups; ++g)
-        if (mark[g] != INFINITY && (at < 0 || mark[g] > best)) { at = g; best = mark[g]; }
-      mark[at] = INFINITY;
+      if (chooser) {
+        const int at = lowest_at(mark, groups);
+        if (lane == 0) mark[at] = -INFINITY;
+      }
+      __syncthreads();
     }
-    for (int g = 0; g < groups; ++g)
-      if (mark[g] != INFINITY)
-        for (int e = g * per; e < (g + 1) * per; ++e) choice[e] = -INFINITY;
+    if (chooser)
+      for (int e = lane; e < n; e += 64)
+        if (mark[e / per] != -INFINITY) choice[e] = -INFINITY;
+    __syncthreads();
   }
   for (int k = 0; k < top; ++k) {
-    int at = 0;
-    float best = choice[0];
-    for (int e = 1; e < n; ++e)
-      if (choice[e] > best) { at = e; best = choice[e]; }
-    ids[(size_t)t * top + k] = at;
-    weights[(size_t)t * top + k] = score[at];
-    choice[at] = -INFINITY;
+    if (chooser) {
+      const int at = lowest_at(choice, n);
+      if (lane == 0) {
+        ids[(size_t)t * top + k] = at;
+        weights[(size_t)t * top + k] = score[at];
+        choice[at] = -INFINITY;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -103,13 +142,17 @@ PLLM_API int pllm_moe_route(int dtype, const void* h, int ld, const float* route
                             int n, int groups, int keep, int top, int* ids, float* weights, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (n <= 0 || groups <= 0 || n % groups || keep <= 0 || keep > groups || top <= 0 || top > (n / groups) * keep) return -2;
-  const size_t lds = (size_t)(2 * n + groups) * sizeof(float);
+  // as many parts of the row as make 16 pieces (1, 2, 4, 8 or 16 parts), none shorter than 64 elements: by the router's
+  // shape alone, so that a token's scores do not depend on the step it is in
+  int segments = 1;
+  while (segments < kRoutePieces && ((n + 7) / 8) * segments < kRoutePieces && width / (2 * segments) >= 64) segments *= 2;
+  const size_t lds = (size_t)(2 * n + groups + segments * n) * sizeof(float);
   if (lds > 48 * 1024) return -2;
-  dim3 grid(num_tokens), block(256);
+  dim3 grid(num_tokens), block(num_tokens >= 128 ? 256 : kRouteThreads);
   if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, lds, stream, (const float*)h, ld, router_w, correction, width, n, groups, keep, top, ids, weights);
+    hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, lds, stream, (const float*)h, ld, router_w, correction, width, n, groups, keep, top, segments, ids, weights);
   else
-    hipLaunchKernelGGL(moe_route_kernel<bf16>, grid, block, lds, stream, (const bf16*)h, ld, router_w, correction, width, n, groups, keep, top, ids, weights);
+    hipLaunchKernelGGL(moe_route_kernel<bf16>, grid, block, lds, stream, (const bf16*)h, ld, router_w, correction, width, n, groups, keep, top, segments, ids, weights);
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -271,7 +314,9 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[u][h][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
   const int k_whole = K & ~31;
-#pragma unroll 2
+  // (a tile of 16 rows streams weights and does little else: eight k-steps of loads under way per wavefront; the large
+  //  tiles hold 4 + 2 operands and 8 accumulators a k-step, and two steps at a time fill the registers)
+#pragma unroll(MT == 1 ? 8 : 2)
   for (int k0 = 0; k0 < k_whole; k0 += 32) {
     moe_bf16x8 a[MT], b[U][W];
 #pragma unroll
@@ -332,11 +377,138 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
   }
 }
 
+// Prompt steps with 128 pairs or more per expert: a workgroup is a tile of 128 rows of one expert times 128 weight rows
+// (gated: 64 of the gate's and the 64 of the up product that belong to them), staged through LDS in k-steps of 64, two
+// buffers deep: every thread fetches eight pieces of 16 bytes of the next step into registers while the matrix cores
+// work on this one, and stores them behind it; one barrier a step.  LDS holds blocks of 16 rows x 32 elements (1 KB) in
+// the operand's order with a row's four pieces XOR-ed by the row's quarter, so that a wavefront's fetch of an operand
+// meets no bank twice.  A wavefront owns 64 x 64 of the tile: 4 + 4 operands and 16 matrix instructions per 32
+// elements of k.  The sums run over ascending k in one accumulator per output, as in the kernel above.
+constexpr int kBigRows = 128;
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __restrict__ rows_in, int ld_in, const bf16* __restrict__ w,
+                                                              const int* __restrict__ tiles, const int* __restrict__ sorted_pair, int top,
+                                                              int n_out, int K, void* __restrict__ out_, int ld_out, int act) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][2][2][8 * 1024];   // [buffer][rows | weights][half of the k-step][8 blocks]
+  const int tile = blockIdx.x;
+  const int expert = tiles[3 * tile], row0 = tiles[3 * tile + 1], nrows = tiles[3 * tile + 2];
+  if (nrows <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.y * (GATED ? 64 : 128);            // this workgroup's first output
+  const bf16* we = w + (size_t)expert * (GATED ? 2 : 1) * n_out * K;
+  // as a loader: pieces tid and tid + 256 of each 8 KB (block p / 64; row (p % 64) / 4 and piece p % 4 of the block)
+  const bf16* a_src[2];
+  const bf16* b_src[2];
+  int put[2], piece_k;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = tid + 256 * i, b = p >> 6, lr = (p & 63) >> 2, lg = p & 3;
+    const int rr = row0 + min(b * 16 + lr, nrows - 1);       // rows past the tile's last repeat it: never stored
+    a_src[i] = rows_in + (size_t)(GATED ? sorted_pair[rr] / top : rr) * ld_in + lg * 8;
+    const int col = GATED ? min(n0 + (b & 3) * 16 + lr, n_out - 1) + (b >> 2) * n_out : min(n0 + b * 16 + lr, n_out - 1);
+    b_src[i] = we + (size_t)col * K + lg * 8;
+    put[i] = b * 1024 + (lr * 4 + (lg ^ ((lr >> 2) & 3))) * 16;
+  }
+  piece_k = (tid & 3) * 8;
+  typedef moe_bf16x8 piece_t;
+  piece_t fetched[2][2][2];                                  // [rows | weights][half][i]
+  const piece_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      const int k = k0 + kh * 32;
+      const bool in = k + piece_k < K;                        // K % 8 == 0: a piece lies inside or outside
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fetched[0][kh][i] = in ? *reinterpret_cast<const piece_t*>(a_src[i] + k) : zero;
+        fetched[1][kh][i] = in ? *reinterpret_cast<const piece_t*>(b_src[i] + k) : zero;
+      }
+    }
+  };
+  auto store = [&](int buf) {
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<piece_t*>(&lds[buf][o][kh][put[i]]) = fetched[o][kh][i];
+  };
+  const int r = lane & 15, g = lane >> 4, wm = wave >> 1, wn = wave & 1;
+  const int take = (r * 4 + (g ^ ((r >> 2) & 3))) * 16;     // where this lane's operand lies in a block
+  int a_blk[4], b_blk[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    a_blk[j] = (wm * 4 + j) * 1024 + take;
+    b_blk[j] = (GATED ? ((j >> 1) * 4 + wn * 2 + (j & 1)) : (wn * 4 + j)) * 1024 + take;
+  }
+  moe_floatx4 acc[4][4];                                     // [weights' block][rows' block]
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[j][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  const int steps = (K + 63) / 64;
+  fetch(0);
+  store(0);
+  __syncthreads();
+  for (int s = 0; s < steps; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < steps) fetch((s + 1) * 64);
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      piece_t a[4], b[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) a[t] = *reinterpret_cast<const piece_t*>(&lds[buf][0][kh][a_blk[t]]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const piece_t*>(&lds[buf][1][kh][b_blk[j]]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j], a[t], acc[j][t], 0, 0, 0);
+    }
+    if (s + 1 < steps) store(buf ^ 1);
+    __syncthreads();
+  }
+  // a lane's four sums: outputs 4 g .. 4 g + 3 of a weights' block, for row r of a rows' block
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = wm * 64 + t * 16 + r;
+    if (row >= nrows) continue;
+    if (GATED) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = n0 + wn * 32 + j * 16 + 4 * g;
+        bf16* o = reinterpret_cast<bf16*>(out_) + (size_t)(row0 + row) * ld_out + col;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col + i < n_out) o[i] = from_f32<bf16>(gate_activation(acc[j][t][i], act) * acc[j + 2][t][i]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = n0 + wn * 64 + j * 16 + 4 * g;
+        if (col >= n_out) continue;
+        float* o = reinterpret_cast<float*>(out_) + (size_t)(row0 + row) * ld_out + col;
+        if (col + 3 < n_out && (ld_out & 3) == 0) {
+          *reinterpret_cast<float4*>(o) = make_float4(acc[j][t][0], acc[j][t][1], acc[j][t][2], acc[j][t][3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (col + i < n_out) o[i] = acc[j][t][i];
+        }
+      }
+    }
+  }
+}
+
 template <bool GATED>
 static void launch_moe_mfma(int tile_rows, int max_tiles, const bf16* rows_in, int ld_in, const bf16* w, const int* tiles,
                             const int* sorted_pair, int top, int n_out, int K, void* out, int ld_out, int act, hipStream_t stream) {
   const int blocks = (n_out + 15) / 16;
-  if (tile_rows >= 64) {
+  if (tile_rows >= kBigRows) {
+    dim3 grid(max_tiles, GATED ? (n_out + 63) / 64 : (n_out + 127) / 128);
+    hipLaunchKernelGGL((moe_expert_tile_kernel<GATED>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
+  } else if (tile_rows >= 64) {
     constexpr int U = GATED ? 1 : 2;
     dim3 grid(max_tiles, (blocks + 4 * U - 1) / (4 * U));
     hipLaunchKernelGGL((moe_expert_mfma_kernel<GATED, 4, U>), grid, dim3(256), 0, stream, rows_in, ld_in, w, tiles, sorted_pair, top, n_out, K, out, ld_out, act);
@@ -354,7 +526,7 @@ PLLM_API int pllm_moe_expert_gemm(int dtype, int gated, const void* rows_in, int
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || K <= 0 || top <= 0 || act < 0 || act >= PLLM_ACT_COUNT) return -2;
   const bool matrix_cores = dtype == PLLM_BF16 && K % 8 == 0 && ld_in % 8 == 0 && ((uintptr_t)rows_in & 15) == 0 && ((uintptr_t)w & 15) == 0;
-  if (tile_rows != kMoeTileRows && !(matrix_cores && tile_rows == kMoeMaxTileRows)) return -2;
+  if (tile_rows != kMoeTileRows && !(matrix_cores && (tile_rows == 64 || tile_rows == kMoeMaxTileRows))) return -2;
   if (matrix_cores) {
     if (gated) launch_moe_mfma<true>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, stream);
     else launch_moe_mfma<false>(tile_rows, max_tiles, (const bf16*)rows_in, ld_in, (const bf16*)w, tiles, sorted_pair, top, n_out, K, out, ld_out, act, stream);

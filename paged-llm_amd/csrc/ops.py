@@ -1487,7 +1487,8 @@ def gate_heads(o: torch.Tensor, gate: torch.Tensor | None, heads: int, dv: int, 
 
 # ------------------------------------------------------------------------------------------- routed experts
 MOE_TILE_ROWS = 16
-MOE_MAX_TILE_ROWS = 64
+MOE_MID_TILE_ROWS = 64
+MOE_MAX_TILE_ROWS = 128
 MOE_MAX_EXPERTS = 1024
 
 
@@ -1513,11 +1514,14 @@ def moe_route(h: torch.Tensor, router_w: torch.Tensor, correction: torch.Tensor 
 
 
 def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, *inner_sizes: int) -> int:
-    """Rows of a tile of the experts' products for a step of ``pairs`` (token, choice) pairs: 64 where the matrix-core
-    kernel runs (bfloat16, every product's inner size a multiple of 8) and an expert gets 32 pairs or more on average,
-    else 16.  It depends on the step's number of tokens only, so a replayed step keeps its choice."""
-    if dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes) and pairs >= 32 * experts:
-        return MOE_MAX_TILE_ROWS
+    """Rows of a tile of the experts' products for a step of ``pairs`` (token, choice) pairs: where the matrix-core
+    kernels run (bfloat16, every product's inner size a multiple of 8) 128 if an expert gets 128 pairs or more on average
+    and 64 if it gets 32 or more, else 16.  It depends on the step's number of tokens only, so a replayed step keeps its choice."""
+    if dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes):
+        if pairs >= 128 * experts:
+            return MOE_MAX_TILE_ROWS
+        if pairs >= 32 * experts:
+            return MOE_MID_TILE_ROWS
     return MOE_TILE_ROWS
 
 
@@ -1528,7 +1532,7 @@ def moe_align(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -
     _on_gpu(ids)
     _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "ids: contiguous int32 [T, top]")
     _need(0 < experts <= MOE_MAX_EXPERTS, f"1 to {MOE_MAX_EXPERTS} experts")
-    _need(tile_rows in (MOE_TILE_ROWS, MOE_MAX_TILE_ROWS), f"tiles of {MOE_TILE_ROWS} or {MOE_MAX_TILE_ROWS} rows")
+    _need(tile_rows in (MOE_TILE_ROWS, MOE_MID_TILE_ROWS, MOE_MAX_TILE_ROWS), f"tiles of {MOE_TILE_ROWS}, {MOE_MID_TILE_ROWS} or {MOE_MAX_TILE_ROWS} rows")
     pairs = ids.numel()
     max_tiles = -(-pairs // tile_rows) + experts
     sorted_pair = torch.empty(pairs, dtype=torch.int32, device=ids.device)
@@ -1550,8 +1554,8 @@ def moe_expert_gemm(rows_in: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor,
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous(), "tiles: int32 [n, 3]")
     pairs = sorted_pair.numel()
     _need(sorted_pair.dtype == torch.int32 and sorted_pair.is_contiguous() and tiles.shape[0] >= -(-pairs // tile_rows), "sorted pairs and their tiles")
-    _need(tile_rows == MOE_TILE_ROWS or (tile_rows == MOE_MAX_TILE_ROWS and rows_in.dtype == torch.bfloat16 and rows_in.shape[1] % 8 == 0
-                                         and rows_in.stride(0) % 8 == 0), "tiles of 64 rows are the matrix-core kernel's")
+    _need(tile_rows == MOE_TILE_ROWS or (tile_rows in (MOE_MID_TILE_ROWS, MOE_MAX_TILE_ROWS) and rows_in.dtype == torch.bfloat16 and rows_in.shape[1] % 8 == 0
+                                         and rows_in.stride(0) % 8 == 0), "tiles of more than 16 rows are the matrix-core kernels'")
     K = rows_in.shape[1]
     N = w.shape[1] // 2 if gated else w.shape[1]
     _need(gated or rows_in.shape[0] == pairs, "the down product takes one row per pair")

@@ -451,7 +451,7 @@ def test_the_router_against_the_plain_choice():
 
 @pytest.mark.parametrize("tokens,width,ff,experts,top", [(5, 64, 32, 3, 2), (200, 96, 40, 4, 3), (300, 128, 72, 2, 1), (131, 40, 100, 5, 5)])
 def test_the_experts_products_on_the_matrix_cores(tokens, width, ff, experts, top):
-    """The bfloat16 kernels of the experts' products (tiles of 16 and of 64 rows; inner sizes with a partial last step
+    """The bfloat16 kernels of the experts' products (tiles of 16, 64 and 128 rows; inner sizes with a partial last step
     of 32; outputs that fill no block of 16) against float64 sums over the same bfloat16 operands, and a pair's row
     bit for bit the same whatever the tile size."""
     from paged_llm_amd.csrc import ops
@@ -461,7 +461,7 @@ def test_the_experts_products_on_the_matrix_cores(tokens, width, ff, experts, to
     w2 = (torch.randn((experts, width, ff), generator=gen) * ff ** -0.5).to(torch.bfloat16).cuda()
     ids = torch.stack([torch.randperm(experts + 1, generator=gen)[:top] for _ in range(tokens)]).to(torch.int32).cuda()   # (expert `experts`: a pass-through one)
     results = []
-    for rows in (ops.MOE_TILE_ROWS, ops.MOE_MAX_TILE_ROWS):
+    for rows in (ops.MOE_TILE_ROWS, ops.MOE_MID_TILE_ROWS, ops.MOE_MAX_TILE_ROWS):
         if rows != ops.MOE_TILE_ROWS and (width % 8 or ff % 8):
             continue                                        # (the plain kernel takes over; it has tiles of 16 rows only)
         sorted_pair, row_of_pair, tiles = ops.moe_align(ids, experts, rows)
@@ -480,8 +480,8 @@ def test_the_experts_products_on_the_matrix_cores(tokens, width, ff, experts, to
         assert torch.allclose(results[-1][0].double(), want_act, rtol=2e-2, atol=2e-2 * float(want_act.abs().max()))
         want_out = torch.einsum("pk,pnk->pn", results[-1][0].double(), w2.cpu().double()[expert])
         assert torch.allclose(results[-1][1].double(), want_out, rtol=1e-4, atol=1e-5 * float(want_out.abs().max()))
-    if len(results) == 2:
-        assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+    for other in results[1:]:
+        assert torch.equal(results[0][0], other[0]) and torch.equal(results[0][1], other[1])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
