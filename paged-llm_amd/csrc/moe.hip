@@ -23,62 +23,103 @@ constexpr int kMoeMaxTileRows = 128;  // ... and of the largest (steps with many
 // corrected score; only experts of the `keep` best groups can be chosen (ties: the lower index wins).
 constexpr int kRouteThreads = 1024, kRoutePieces = 16;   // threads of a workgroup in steps of few tokens; pieces the products are cut into
 
-template <typename T>
+template <typename T, int TOK>
 __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ router_w,
-                                                                  const float* __restrict__ correction, int width, int n, int groups, int keep,
-                                                                  int top, int segments, int* __restrict__ ids, float* __restrict__ weights) {
+                                                                  const float* __restrict__ correction, int num_tokens, int width, int n,
+                                                                  int groups, int keep, int top, int segments, int* __restrict__ ids,
+                                                                  float* __restrict__ weights) {
   extern __shared__ float lds[];
-  float* score = lds;            // [n]  router outputs, then scores
-  float* choice = lds + n;       // [n]  score + correction, -inf once taken or shut out
-  float* mark = lds + 2 * n;     // [groups]
-  float* part = mark + groups;   // [segments][n]  sums over a segment of the row
-  const int t = blockIdx.x;
+  const int per_token = 2 * n + groups + segments * n;       // floats of LDS that one token has
+  const int t0 = blockIdx.x * TOK;                           // this workgroup's tokens: t0 .. t0 + TOK - 1
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const T* row = h + (size_t)t * ld;
-  // The router's products.  A piece of work is eight router rows times one of `segments` equal parts of the token's
-  // row, and the wavefronts (16 in steps of few tokens, 4 in others) take the pieces in turn: one pass over the part with eight independent loads and sums
-  // per element, several elements under way (few tokens, a router matrix that the experts' weights have pushed out of
-  // the caches since the last layer: what counts is how few loads wait for one another).  A router output is the sum
-  // of its parts in ascending order, each part summed lane by lane and then over the wavefront.
+  const T* row[TOK];
+#pragma unroll
+  for (int k = 0; k < TOK; ++k) row[k] = h + (size_t)min(t0 + k, num_tokens - 1) * ld;     // (tokens past the last repeat it: not stored)
+  // The router's products.  A piece of work is eight router rows times one of `segments` equal parts of the tokens'
+  // rows, and the wavefronts (16 in steps of few tokens, 4 in others) take the pieces in turn: one pass over the part
+  // with eight independent loads and sums per element and token, several elements under way (few tokens, a router matrix
+  // that the experts' weights have pushed out of the caches since the last layer: what counts is how few loads wait for
+  // one another; many tokens: a router element is fetched once for TOK of them).  A router output is the sum of its
+  // parts in ascending order, each part summed lane by lane and then over the wavefront, whatever TOK is.
   const int batches = (n + 7) / 8;
   const int seg = ((width + segments - 1) / segments + 63) & ~63;
   for (int piece = wave; piece < batches * segments; piece += (int)(blockDim.x >> 6)) {
     const int e0 = (piece / segments) * 8, sg = piece % segments;
     const int from = sg * seg, to = min(width, from + seg);
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const float* w = router_w + (size_t)e0 * width;
-    if (e0 + 8 <= n) {
-#pragma unroll 8
-      for (int i = from + lane; i < to; i += 64) {
-        const float x = to_f32(row[i]);
+    float acc[8][TOK];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = fmaf(x, w[(size_t)j * width + i], acc[j]);
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int k = 0; k < TOK; ++k) acc[j][k] = 0.f;
+    const float* w = router_w + (size_t)e0 * width;
+    if (TOK == 1 && e0 + 8 <= n) {
+      // every load of eight elements' worth asked for before the first sum: 72 loads under way, one trip to memory
+      for (int i0 = from + lane; i0 < to; i0 += 8 * 64) {
+        float x[8], wv[8][8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = min(i0 + u * 64, to - 1);
+          x[u] = i0 + u * 64 < to ? to_f32(row[0][i]) : 0.f;      // (an element past the part counts as zero times a valid weight)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) wv[u][j] = w[(size_t)j * width + i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[j][0] = fmaf(x[u], wv[u][j], acc[j][0]);
+      }
+    } else if (e0 + 8 <= n) {
+#pragma unroll 2
+      for (int i = from + lane; i < to; i += 64) {
+        float x[TOK];
+#pragma unroll
+        for (int k = 0; k < TOK; ++k) x[k] = to_f32(row[k][i]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float wj = w[(size_t)j * width + i];
+#pragma unroll
+          for (int k = 0; k < TOK; ++k) acc[j][k] = fmaf(x[k], wj, acc[j][k]);
+        }
       }
     } else {
       for (int i = from + lane; i < to; i += 64) {
-        const float x = to_f32(row[i]);
+        float x[TOK];
+#pragma unroll
+        for (int k = 0; k < TOK; ++k) x[k] = to_f32(row[k][i]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-          if (e0 + j < n) acc[j] = fmaf(x, w[(size_t)j * width + i], acc[j]);
+          if (e0 + j < n) {
+            const float wj = w[(size_t)j * width + i];
+#pragma unroll
+            for (int k = 0; k < TOK; ++k) acc[j][k] = fmaf(x[k], wj, acc[j][k]);
+          }
       }
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float total = wave_sum(acc[j]);
-      if (lane == 0 && e0 + j < n) part[sg * n + e0 + j] = total;
-    }
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int k = 0; k < TOK; ++k) {
+        const float total = wave_sum(acc[j][k]);
+        if (lane == 0 && e0 + j < n) lds[k * per_token + 2 * n + groups + sg * n + e0 + j] = total;
+      }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < n; e += blockDim.x) {
+  for (int i = threadIdx.x; i < TOK * n; i += blockDim.x) {
+    const int k = i / n, e = i - k * n;
+    const float* part = lds + k * per_token + 2 * n + groups;
     float total = part[e];
     for (int sg = 1; sg < segments; ++sg) total += part[sg * n + e];
-    score[e] = total;
+    lds[k * per_token + e] = total;
   }
   __syncthreads();
-  // The choice, by the first wavefront (the others keep it company at the barriers): lane l looks after router outputs
-  // l, l + 64, ...; a largest element is found by a maximum over the wavefront and then the lowest index that holds it
-  // (ties: the lower index wins).
-  const bool chooser = wave == 0;
+  // The choice: wavefront k makes token t0 + k's (the others keep them company at the barriers).
+  const int t = t0 + wave;
+  const bool chooser = wave < TOK && t < num_tokens;
+  float* score = lds + (wave < TOK ? wave : 0) * per_token;   // [n]  router outputs, then scores
+  float* choice = score + n;                                  // [n]  score + correction, -inf once taken or shut out
+  float* mark = score + 2 * n;                                // [groups]
+  // Lane l looks after router outputs l, l + 64, ...; a largest element is found by a maximum over the wavefront and
+  // then the lowest index that holds it (ties: the lower index wins).
   auto lowest_at = [&](const float* values, int count) {
     float mine = -INFINITY;
     for (int e = lane; e < count; e += 64) mine = fmaxf(mine, values[e]);
@@ -146,13 +187,16 @@ PLLM_API int pllm_moe_route(int dtype, const void* h, int ld, const float* route
   // shape alone, so that a token's scores do not depend on the step it is in
   int segments = 1;
   while (segments < kRoutePieces && ((n + 7) / 8) * segments < kRoutePieces && width / (2 * segments) >= 64) segments *= 2;
-  const size_t lds = (size_t)(2 * n + groups + segments * n) * sizeof(float);
+  const size_t lds_one = (size_t)(2 * n + groups + segments * n) * sizeof(float);
+  const bool many = num_tokens >= 128 && 4 * lds_one <= 48 * 1024;   // four tokens to a workgroup of four wavefronts, or one to sixteen
+  const size_t lds = lds_one * (many ? 4 : 1);
   if (lds > 48 * 1024) return -2;
-  dim3 grid(num_tokens), block(num_tokens >= 128 ? 256 : kRouteThreads);
-  if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, lds, stream, (const float*)h, ld, router_w, correction, width, n, groups, keep, top, segments, ids, weights);
-  else
-    hipLaunchKernelGGL(moe_route_kernel<bf16>, grid, block, lds, stream, (const bf16*)h, ld, router_w, correction, width, n, groups, keep, top, segments, ids, weights);
+#define PLLM_ROUTE(T, TOK, THREADS)                                                                                              \
+  hipLaunchKernelGGL((moe_route_kernel<T, TOK>), dim3((num_tokens + TOK - 1) / TOK), dim3(THREADS), lds, stream, (const T*)h, ld, \
+                     router_w, correction, num_tokens, width, n, groups, keep, top, segments, ids, weights)
+  if (dtype == PLLM_F32) { if (many) PLLM_ROUTE(float, 4, 256); else PLLM_ROUTE(float, 1, kRouteThreads); }
+  else { if (many) PLLM_ROUTE(bf16, 4, 256); else PLLM_ROUTE(bf16, 1, kRouteThreads); }
+#undef PLLM_ROUTE
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -314,10 +358,37 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[u][h][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
   const int k_whole = K & ~31;
-  // (a tile of 16 rows streams weights and does little else: eight k-steps of loads under way per wavefront; the large
-  //  tiles hold 4 + 2 operands and 8 accumulators a k-step, and two steps at a time fill the registers)
-#pragma unroll(MT == 1 ? 8 : 2)
-  for (int k0 = 0; k0 < k_whole; k0 += 32) {
+  int k_done = 0;
+  if (MT == 1) {
+    // A tile of 16 rows streams weights and does little else.  Two k-steps at a time, with a lane holding 16
+    // neighbouring elements of its row (32 bytes; four lanes read a whole line of 128) of which the first eight feed one
+    // matrix instruction and the last eight the next: rows and weights are cut the same way, so the 64 products of an
+    // output are the same ones, summed in two other halves than with 8 + 8 elements 32 apart.  Four such pairs of
+    // steps are under way per wavefront.
+    const int k_pairs = K & ~63;
+#pragma unroll 4
+    for (int k0 = 0; k0 < k_pairs; k0 += 64) {
+      moe_bf16x8 a[2], b[U][W][2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        a[half] = *reinterpret_cast<const moe_bf16x8*>(a_ptr[0] + k0 + 8 * g + 8 * half);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int h = 0; h < W; ++h) b[u][h][half] = *reinterpret_cast<const moe_bf16x8*>(w_ptr[u][h] + k0 + 8 * g + 8 * half);
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int h = 0; h < W; ++h) acc[u][h][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[u][h][half], a[half], acc[u][h][0], 0, 0, 0);
+    }
+    k_done = k_pairs;
+  }
+  // (the large tiles hold 4 + 2 operands and 8 accumulators a k-step, and two steps at a time fill the registers)
+#pragma unroll 2
+  for (int k0 = k_done; k0 < k_whole; k0 += 32) {
     moe_bf16x8 a[MT], b[U][W];
 #pragma unroll
     for (int t = 0; t < MT; ++t) a[t] = *reinterpret_cast<const moe_bf16x8*>(a_ptr[t] + k0);
