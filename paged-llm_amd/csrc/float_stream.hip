@@ -232,11 +232,114 @@ __global__ __launch_bounds__(256) void rms_sandwich_kernel(const float* __restri
   }
 }
 
+// The same with a branch, for rows of up to 4,096 elements that 256 threads hold in registers (16 each): everything a
+// row needs (branch and bias, the stream's row, both weights) is asked for before the first sum, so the kernel waits
+// for memory once where the one above waits three times (decode steps: the weights have left the caches since the last
+// layer).  Elements, partial sums and their order are the ones of the kernel above.  The branch may still be a sum of
+// experts' rows (`sum.expert_out` set): branch[r][i] = sum over k < top, in order, of weights[r, k] * (row_of_pair[r, k]
+// >= 0 ? expert_out[row_of_pair[r, k]][i] : h[r][i]), formed here instead of by a kernel of its own.
+struct ChoiceSum {
+  const float* expert_out; const void* h; long ld_h; const int* row_of_pair; const float* weights; int top;
+};
+constexpr int kHeldPerThread = 16, kHeldThreads = 256;
+
+template <typename TO, typename TH>
+__global__ __launch_bounds__(kHeldThreads) void rms_sandwich_held_kernel(const float* __restrict__ branch, const ChoiceSum sum,
+                                                                         const float* __restrict__ bias, const float* __restrict__ w_branch,
+                                                                         float mult, float* stream, const float* __restrict__ w_next, float eps,
+                                                                         TO* __restrict__ rows, long rows_stride, int hidden) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  float* s = stream + (size_t)r * hidden;
+  float f[kHeldPerThread], sv[kHeldPerThread], wb[kHeldPerThread], wn[kHeldPerThread];
+#pragma unroll
+  for (int j = 0; j < kHeldPerThread; ++j) {
+    const int i = tid + kHeldThreads * j;
+    const bool in = i < hidden;
+    sv[j] = in ? s[i] : 0.f;
+    wb[j] = in ? w_branch[i] : 0.f;
+    wn[j] = (in && w_next) ? w_next[i] : 1.f;
+    f[j] = (in && !sum.expert_out) ? branch[(size_t)r * hidden + i] : 0.f;
+  }
+  if (sum.expert_out) {
+    const TH* own = reinterpret_cast<const TH*>(sum.h) + (size_t)r * sum.ld_h;
+    for (int k = 0; k < sum.top; ++k) {
+      const int row = sum.row_of_pair[(size_t)r * sum.top + k];
+      const float wk = sum.weights[(size_t)r * sum.top + k];
+      const float* e = sum.expert_out + (size_t)(row >= 0 ? row : 0) * hidden;
+#pragma unroll
+      for (int j = 0; j < kHeldPerThread; ++j) {
+        const int i = tid + kHeldThreads * j;
+        if (i < hidden) f[j] = fmaf(wk, row >= 0 ? e[i] : to_f32(own[i]), f[j]);
+      }
+    }
+  }
+  float bsq = 0.f;
+#pragma unroll
+  for (int j = 0; j < kHeldPerThread; ++j) {
+    const int i = tid + kHeldThreads * j;
+    if (i < hidden) {
+      if (bias) f[j] += bias[i];
+      bsq = fmaf(f[j], f[j], bsq);
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(bsq, scratch) / (float)hidden + eps);
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < kHeldPerThread; ++j) {
+    const int i = tid + kHeldThreads * j;
+    if (i < hidden) {
+      const float y = sv[j] + mult * (f[j] * inv * wb[j]);
+      s[i] = y;
+      sv[j] = y;
+      sq = fmaf(y, y, sq);
+    }
+  }
+  if (!rows) return;
+  TO* out = rows + (size_t)r * rows_stride;
+  const float inv_next = w_next ? 1.f / sqrtf(block_sum(sq, scratch) / (float)hidden + eps) : 1.f;
+#pragma unroll
+  for (int j = 0; j < kHeldPerThread; ++j) {
+    const int i = tid + kHeldThreads * j;
+    if (i < hidden) out[i] = from_f32<TO>(w_next ? sv[j] * inv_next * wn[j] : sv[j]);
+  }
+}
+
+template <typename TO>
+static void launch_sandwich_held(int h_dtype, const float* branch, const ChoiceSum& sum, const float* bias, const float* w_branch, float mult,
+                                 float* stream, const float* w_next, float eps, void* rows, long rows_stride, int num_rows, int hidden,
+                                 hipStream_t stream_) {
+  if (h_dtype == PLLM_F32)
+    hipLaunchKernelGGL((rms_sandwich_held_kernel<TO, float>), dim3(num_rows), dim3(kHeldThreads), 0, stream_, branch, sum, bias, w_branch, mult,
+                       stream, w_next, eps, (TO*)rows, rows_stride, hidden);
+  else
+    hipLaunchKernelGGL((rms_sandwich_held_kernel<TO, bf16>), dim3(num_rows), dim3(kHeldThreads), 0, stream_, branch, sum, bias, w_branch, mult,
+                       stream, w_next, eps, (TO*)rows, rows_stride, hidden);
+}
+
+// A branch that is a sum of experts' rows (see above); rows of up to 4,096 elements.
+PLLM_API int pllm_rms_sandwich_sum(int out_dtype, int h_dtype, const float* expert_out, const void* h, long ld_h, const int* row_of_pair,
+                                   const float* weights, int top, const float* bias, const float* w_branch, float mult, float* stream,
+                                   const float* w_next, float eps, void* rows, long rows_stride, int num_rows, int hidden, hipStream_t stream_) {
+  if (num_rows <= 0) return 0;
+  if (hidden <= 0 || hidden > kHeldPerThread * kHeldThreads || !stream || !w_branch || !expert_out || !h || !row_of_pair || !weights || top <= 0) return -2;
+  const ChoiceSum sum{expert_out, h, ld_h, row_of_pair, weights, top};
+  if (out_dtype == PLLM_F32) launch_sandwich_held<float>(h_dtype, nullptr, sum, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+  else launch_sandwich_held<bf16>(h_dtype, nullptr, sum, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+  PLLM_RETURN_LAST_ERROR();
+}
+
 PLLM_API int pllm_rms_sandwich(int out_dtype, const float* branch, const float* bias, const float* w_branch, float mult, float* stream,
                                const int* row_index, const float* w_next, float eps, void* rows, long rows_stride, int num_rows,
                                int hidden, hipStream_t stream_) {
   if (num_rows <= 0) return 0;
   if (hidden <= 0 || !stream || (branch && !w_branch)) return -2;
+  if (branch && hidden <= kHeldPerThread * kHeldThreads) {
+    const ChoiceSum none{nullptr, nullptr, 0, nullptr, nullptr, 0};
+    if (out_dtype == PLLM_F32) launch_sandwich_held<float>(PLLM_F32, branch, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+    else launch_sandwich_held<bf16>(PLLM_F32, branch, none, bias, w_branch, mult, stream, w_next, eps, rows, rows_stride, num_rows, hidden, stream_);
+    PLLM_RETURN_LAST_ERROR();
+  }
   const size_t lds = (size_t)(hidden + 16) * sizeof(float);
   dim3 grid(num_rows), block(256);
 #define PLLM_SW(TO)                                                                                                        \

@@ -1375,20 +1375,63 @@ def latent_attention(q: torch.Tensor, rank: int, rot: int, k_pages: torch.Tensor
 
 
 # ------------------------------------------------------------------------------------------- norms on both sides of a branch
+SANDWICH_HELD_MAX = 4096      # rows that the norm-add-norm kernel holds in registers
+
+
+class ChoiceSum:
+    """The result of routed experts before its last step: per token the sum, over its choices in order, of weight times
+    the pair's row of ``expert_out`` (float32 [pairs, width]) or, where ``row_of_pair`` is -1, the token's own row of
+    ``h``.  ``rows()`` forms it (``moe_combine``); ``rms_sandwich`` takes it as a branch and forms it in its own kernel."""
+
+    def __init__(self, expert_out: torch.Tensor, h: torch.Tensor, row_of_pair: torch.Tensor, weights: torch.Tensor):
+        self.expert_out, self.h, self.row_of_pair, self.weights = expert_out, h, row_of_pair, weights
+
+    def rows(self) -> torch.Tensor:
+        return moe_combine(self.expert_out, self.h, self.row_of_pair, self.weights)
+
+    def checked(self, rows: int, width: int):
+        e, h, rp, wt = self.expert_out, self.h, self.row_of_pair, self.weights
+        _on_gpu(e, h, rp, wt)
+        _need(wt.dtype == torch.float32 and wt.dim() == 2 and wt.shape[0] == rows and wt.is_contiguous(), "weights: float32 [rows, top]")
+        top = wt.shape[1]
+        _need(e.dtype == torch.float32 and e.shape == (rows * top, width) and e.is_contiguous(), f"expert outputs: float32 [{rows * top}, {width}]")
+        _need(h.dim() == 2 and h.shape == (rows, width) and h.stride(1) == 1 and h.dtype in (torch.float32, torch.bfloat16), "the tokens' rows: [rows, width]")
+        _need(rp.dtype == torch.int32 and rp.numel() == rows * top and rp.is_contiguous(), "row_of_pair: int32 [rows * top]")
+        return e, h, rp, wt
+
+
 def rms_sandwich(stream: torch.Tensor, branch: torch.Tensor | None, w_branch: torch.Tensor | None, mult: float, eps: float,
                  w_next: torch.Tensor | None = None, out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
                  bias: torch.Tensor | None = None, row_index: torch.Tensor | None = None) -> torch.Tensor | None:
-    """RMS norms around a float32 residual stream, all in float.  With ``branch`` (float32 rows like the stream):
+    """RMS norms around a float32 residual stream, all in float.  With ``branch`` (float32 rows like the stream, or a
+    ``ChoiceSum``: a weighted sum of experts' rows that the kernel forms itself):
     stream += mult * rms_norm(branch + bias) * w_branch, in place.  Then, when ``out`` or ``out_dtype`` is given, the
     rows of the stream as it is now are returned in that type: normed and times ``w_next``, or as they are when
     ``w_next`` is None.  ``out`` may be a view with a row stride of its own (unit inner stride).  Without a branch
     ``row_index`` (int32) picks the rows of the stream; nothing is written to the stream then."""
-    _on_gpu(stream, branch, w_branch, w_next, out, bias, row_index)
+    _on_gpu(stream, None if isinstance(branch, ChoiceSum) else branch, w_branch, w_next, out, bias, row_index)
     _need(stream.dtype == torch.float32 and stream.dim() == 2 and stream.is_contiguous(), "the stream is contiguous float32 [rows, hidden]")
     rows, H = stream.shape
     _need((H + 16) * 4 <= min(_max_lds_bytes(stream.device), 160 * 1024), f"the norm kernel stages one row in LDS: hidden size {H} is above its limit")
     for t, what in ((w_branch, "w_branch"), (w_next, "w_next"), (bias, "bias")):
         _need(t is None or (t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()), f"{what} must be float32 [{H}]")
+    if isinstance(branch, ChoiceSum):
+        if H > SANDWICH_HELD_MAX:
+            branch = branch.rows()                          # (rows too long for the kernel that holds them in registers)
+        else:
+            _need(row_index is None and w_branch is not None, "a branch comes with its norm's weight, and no rows are picked")
+            if out is None and out_dtype is not None:
+                out = torch.empty((rows, H), dtype=out_dtype, device=stream.device)
+            if out is not None:
+                _need(out.dim() == 2 and out.shape == (rows, H) and out.stride(1) == 1, f"the rows' output is [{rows}, {H}] with unit inner stride")
+            e, h, rp, wt = branch.checked(rows, H)
+            _check(_fn("float_stream.hip", "pllm_rms_sandwich_sum",
+                       signature=[c_int, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                  c_float, c_void_p, c_long, c_int, c_int, c_void_p])(
+                dtype_code(out.dtype) if out is not None else F32, dtype_code(h.dtype), _ptr(e), _ptr(h), h.stride(0), _ptr(rp), _ptr(wt), wt.shape[1],
+                _ptr(bias), _ptr(w_branch), c_float(mult), _ptr(stream), _ptr(w_next), c_float(eps), _ptr(out),
+                out.stride(0) if out is not None else 0, rows, H, _stream()), "rms_sandwich_sum")
+            return out
     if branch is not None:
         _need(branch.dtype == torch.float32 and branch.shape == stream.shape and branch.is_contiguous() and w_branch is not None,
               "a branch is contiguous float32 rows like the stream, with its norm's weight")

@@ -143,7 +143,9 @@ class SandwichNormBlock(Block):
         bias = getattr(p["mixer"], "output_bias", None)
         if self.has_feed_forward:
             h = p["mixer_out_norm"].add_to(x, a, self.mult, bias=bias, then=p["feed_forward_norm"])
+            ctx.branch_sum_ok = True      # a feed-forward may hand over a sum that the norm's kernel forms (``ops.ChoiceSum``)
             m = p["feed_forward"].forward(h, ctx)
+            ctx.branch_sum_ok = False
             a, bias, last = m, getattr(p["feed_forward"], "output_bias", None), p["feed_forward_out_norm"]
         else:
             last = p["mixer_out_norm"]

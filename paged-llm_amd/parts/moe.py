@@ -79,6 +79,8 @@ class RoutedExperts(FeedForward):
         sorted_pair, row_of_pair, tiles = ops.moe_align(ids, self.experts, rows)
         act = ops.moe_expert_gemm(h, self.w_gate_up, tiles, sorted_pair, self.top, True, self.activation, tile_rows=rows)
         out = ops.moe_expert_gemm(act, self.w_down, tiles, sorted_pair, self.top, False, tile_rows=rows)
+        if getattr(ctx, "float_branch", False) and getattr(ctx, "branch_sum_ok", False):
+            return ops.ChoiceSum(out, h, row_of_pair, weights)      # whoever norms the branch forms the sum in its kernel
         y = ops.moe_combine(out, h, row_of_pair, weights)
         if getattr(ctx, "float_branch", False):
             return y
