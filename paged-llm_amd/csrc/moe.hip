@@ -36,7 +36,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
 #pragma unroll
   for (int k = 0; k < TOK; ++k) row[k] = h + (size_t)min(t0 + k, num_tokens - 1) * ld;     // (tokens past the last repeat it: not stored)
   // The router's products.  A piece of work is eight router rows times one of `segments` equal parts of the tokens'
-  // rows, and the wavefronts (16 in steps of few tokens, 4 in others) take the pieces in turn: one pass over the part
+  // rows, and the wavefronts (16 for one token; 4 or 8 where a workgroup has as many tokens) take the pieces in turn: one pass over the part
   // with eight independent loads and sums per element and token, several elements under way (few tokens, a router matrix
   // that the experts' weights have pushed out of the caches since the last layer: what counts is how few loads wait for
   // one another; many tokens: a router element is fetched once for TOK of them).  A router output is the sum of its
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
           for (int j = 0; j < 8; ++j) acc[j][0] = fmaf(x[u], wv[u][j], acc[j][0]);
       }
     } else if (e0 + 8 <= n) {
-#pragma unroll 2
+#pragma unroll(TOK >= 8 ? 1 : 2)
       for (int i = from + lane; i < to; i += 64) {
         float x[TOK];
 #pragma unroll
@@ -188,14 +188,15 @@ PLLM_API int pllm_moe_route(int dtype, const void* h, int ld, const float* route
   int segments = 1;
   while (segments < kRoutePieces && ((n + 7) / 8) * segments < kRoutePieces && width / (2 * segments) >= 64) segments *= 2;
   const size_t lds_one = (size_t)(2 * n + groups + segments * n) * sizeof(float);
-  const bool many = num_tokens >= 128 && 4 * lds_one <= 48 * 1024;   // four tokens to a workgroup of four wavefronts, or one to sixteen
-  const size_t lds = lds_one * (many ? 4 : 1);
-  if (lds > 48 * 1024) return -2;
+  // tokens to a workgroup (one wavefront each for the choice): 8 in steps of 512 tokens and more, 4 from 128 on, else one
+  // token to sixteen wavefronts
+  const int tok = (num_tokens >= 512 && 8 * lds_one <= 48 * 1024) ? 8 : (num_tokens >= 128 && 4 * lds_one <= 48 * 1024) ? 4 : 1;
+  const size_t lds = lds_one * tok;
 #define PLLM_ROUTE(T, TOK, THREADS)                                                                                              \
   hipLaunchKernelGGL((moe_route_kernel<T, TOK>), dim3((num_tokens + TOK - 1) / TOK), dim3(THREADS), lds, stream, (const T*)h, ld, \
                      router_w, correction, num_tokens, width, n, groups, keep, top, segments, ids, weights)
-  if (dtype == PLLM_F32) { if (many) PLLM_ROUTE(float, 4, 256); else PLLM_ROUTE(float, 1, kRouteThreads); }
-  else { if (many) PLLM_ROUTE(bf16, 4, 256); else PLLM_ROUTE(bf16, 1, kRouteThreads); }
+  if (dtype == PLLM_F32) { if (tok == 8) PLLM_ROUTE(float, 8, 512); else if (tok == 4) PLLM_ROUTE(float, 4, 256); else PLLM_ROUTE(float, 1, kRouteThreads); }
+  else { if (tok == 8) PLLM_ROUTE(bf16, 8, 512); else if (tok == 4) PLLM_ROUTE(bf16, 4, 256); else PLLM_ROUTE(bf16, 1, kRouteThreads); }
 #undef PLLM_ROUTE
   PLLM_RETURN_LAST_ERROR();
 }
@@ -450,12 +451,20 @@ __global__ __launch_bounds__(256) void moe_expert_mfma_kernel(const bf16* __rest
 
 // Prompt steps with 128 pairs or more per expert: a workgroup is a tile of 128 rows of one expert times 128 weight rows
 // (gated: 64 of the gate's and the 64 of the up product that belong to them), staged through LDS in k-steps of 64, two
-// buffers deep: every thread fetches eight pieces of 16 bytes of the next step into registers while the matrix cores
-// work on this one, and stores them behind it; one barrier a step.  LDS holds blocks of 16 rows x 32 elements (1 KB) in
+// buffers deep: every thread fetches eight pieces of 16 bytes of the steps ahead into registers while the matrix cores
+// work on this one, and stores a step's pieces behind the products of the step before; one barrier a step, which waits
+// for LDS stores only.  LDS holds blocks of 16 rows x 32 elements (1 KB) in
 // the operand's order with a row's four pieces XOR-ed by the row's quarter, so that a wavefront's fetch of an operand
 // meets no bank twice.  A wavefront owns 64 x 64 of the tile: 4 + 4 operands and 16 matrix instructions per 32
 // elements of k.  The sums run over ascending k in one accumulator per output, as in the kernel above.
 constexpr int kBigRows = 128;
+
+// A workgroup barrier that waits for this wavefront's LDS stores and nothing else: loads from memory that are under way
+// stay under way across it (a barrier with a fence in front waits for them all, and with them for the steps asked for ahead).
+__device__ __forceinline__ void tile_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xC07F);                         // lgkmcnt(0); vmcnt and expcnt as they are
+  asm volatile("s_barrier" ::: "memory");
+}
 
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __restrict__ rows_in, int ld_in, const bf16* __restrict__ w,
@@ -483,27 +492,30 @@ __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __rest
   }
   piece_k = (tid & 3) * 8;
   typedef moe_bf16x8 piece_t;
-  piece_t fetched[2][2][2];                                  // [rows | weights][half][i]
+  // Three sets of registers: the pieces of step s + 1 were asked for two steps ago and go into LDS behind the products
+  // of step s, those of steps s + 2 and s + 3 are under way.  (Measured the same as one step under way: what bounds the
+  // kernel is the 32 KB that a workgroup draws from the L2 per step, 1.7 GB a call at width 2,048 and 2,048 tokens.)
+  piece_t fetched[3][2][2][2];                               // [set][rows | weights][half][i]
   const piece_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  auto fetch = [&](int k0) {
+  auto fetch = [&](piece_t (&set)[2][2][2], int k0) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
       const int k = k0 + kh * 32;
       const bool in = k + piece_k < K;                        // K % 8 == 0: a piece lies inside or outside
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        fetched[0][kh][i] = in ? *reinterpret_cast<const piece_t*>(a_src[i] + k) : zero;
-        fetched[1][kh][i] = in ? *reinterpret_cast<const piece_t*>(b_src[i] + k) : zero;
+        set[0][kh][i] = in ? *reinterpret_cast<const piece_t*>(a_src[i] + k) : zero;
+        set[1][kh][i] = in ? *reinterpret_cast<const piece_t*>(b_src[i] + k) : zero;
       }
     }
   };
-  auto store = [&](int buf) {
+  auto store = [&](const piece_t (&set)[2][2][2], int buf) {
 #pragma unroll
     for (int o = 0; o < 2; ++o)
 #pragma unroll
       for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<piece_t*>(&lds[buf][o][kh][put[i]]) = fetched[o][kh][i];
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<piece_t*>(&lds[buf][o][kh][put[i]]) = set[o][kh][i];
   };
   const int r = lane & 15, g = lane >> 4, wm = wave >> 1, wn = wave & 1;
   const int take = (r * 4 + (g ^ ((r >> 2) & 3))) * 16;     // where this lane's operand lies in a block
@@ -518,13 +530,7 @@ __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __rest
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[j][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
-  const int steps = (K + 63) / 64;
-  fetch(0);
-  store(0);
-  __syncthreads();
-  for (int s = 0; s < steps; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < steps) fetch((s + 1) * 64);
+  auto products = [&](int buf) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
       piece_t a[4], b[4];
@@ -537,9 +543,27 @@ __global__ __launch_bounds__(256) void moe_expert_tile_kernel(const bf16* __rest
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j], a[t], acc[j][t], 0, 0, 0);
     }
-    if (s + 1 < steps) store(buf ^ 1);
-    __syncthreads();
+  };
+  const int steps = (K + 63) / 64;
+  fetch(fetched[0], 0);
+  if (steps > 1) fetch(fetched[1], 64);
+  if (steps > 2) fetch(fetched[2], 128);
+  store(fetched[0], 0);
+  tile_barrier();
+  // step s: ask for step s + 3 into the set that step s came from, multiply step s, put step s + 1 into the other buffer
+#define PLLM_TILE_STEP(S, FREE_SET, NEXT_SET)                         \
+  {                                                                   \
+    if ((S) + 3 < steps) fetch(fetched[FREE_SET], ((S) + 3) * 64);    \
+    products((S) & 1);                                                \
+    if ((S) + 1 < steps) store(fetched[NEXT_SET], ((S) + 1) & 1);     \
+    tile_barrier();                                                  \
   }
+  for (int s3 = 0; s3 < steps; s3 += 3) {
+    PLLM_TILE_STEP(s3, 0, 1)
+    if (s3 + 1 < steps) PLLM_TILE_STEP(s3 + 1, 1, 2)
+    if (s3 + 2 < steps) PLLM_TILE_STEP(s3 + 2, 2, 0)
+  }
+#undef PLLM_TILE_STEP
   // a lane's four sums: outputs 4 g .. 4 g + 3 of a weights' block, for row r of a rows' block
 #pragma unroll
   for (int t = 0; t < 4; ++t) {

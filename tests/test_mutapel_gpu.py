@@ -437,7 +437,7 @@ def test_the_router_against_the_plain_choice():
     from paged_llm_amd.csrc import ops
     gen = torch.Generator().manual_seed(3)
     for n, groups, keep, top, shift in [(12, 4, 2, 3, -2.0), (16, 4, 1, 4, 0.0), (18, 3, 2, 5, -0.5), (7, 7, 3, 3, 0.3), (8, 1, 1, 8, -1.0), (6, 2, 2, 1, 0.0)]:
-        h = torch.randn((203, 40), generator=gen)             # (steps of 128 tokens and more: four tokens to a workgroup)
+        h = torch.randn((203 if n % 2 else 515, 40), generator=gen)     # (steps of 128 and of 512 tokens and more: four and eight tokens to a workgroup)
         w = torch.randn((n, 40), generator=gen) * 0.4
         corr = torch.randn((n,), generator=gen) * 0.2 + shift
         r = {"groups": {"count": groups, "keep": keep}, "top": top}
