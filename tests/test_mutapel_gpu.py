@@ -489,6 +489,36 @@ def test_the_experts_products_on_the_matrix_cores(tokens, width, ff, experts, to
         assert torch.allclose(results[0][0].float(), results[1][0].float(), rtol=2 ** -7, atol=1e-3 * float(results[1][0].float().abs().max()))
 
 
+@pytest.mark.parametrize("width", [40, 96, 2048, 4100])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_norm_forms_the_experts_sum_itself(width, dtype):
+    """The kernel that norms a branch, adds it to the stream and norms the stream for the next reader, given the
+    experts' rows, places and weights instead of their finished sum: bit for bit what it gives after ``moe_combine``
+    (rows held in registers up to 4,096 elements; longer rows take the sum first), and close to float64."""
+    from paged_llm_amd.csrc import ops
+    gen = torch.Generator().manual_seed(width)
+    tokens, top = 7, 3
+    stream = torch.randn((tokens, width), generator=gen).cuda()
+    expert_out = torch.randn((tokens * top, width), generator=gen).cuda()
+    h = torch.randn((tokens, width), generator=gen).to(dtype).cuda()
+    places = torch.randperm(tokens * top, generator=gen).to(torch.int32)
+    places[torch.tensor([1, 5, 6, 20])] = -1                                 # (choices that hand the token's own row back)
+    places = places.cuda()
+    weights = torch.rand((tokens, top), generator=gen).cuda()
+    w_branch, w_next = (torch.randn((width,), generator=gen) * 0.1 + 1.0).cuda(), (torch.randn((width,), generator=gen) * 0.1 + 1.0).cuda()
+    a, b = stream.clone(), stream.clone()
+    rows_a = ops.rms_sandwich(a, ops.ChoiceSum(expert_out, h, places, weights), w_branch, 0.4, 1e-5, w_next=w_next, out_dtype=dtype)
+    rows_b = ops.rms_sandwich(b, ops.ChoiceSum(expert_out, h, places, weights).rows(), w_branch, 0.4, 1e-5, w_next=w_next, out_dtype=dtype)
+    assert torch.equal(a, b) and torch.equal(rows_a, rows_b)
+    picked = torch.where(places.view(tokens, top, 1).cpu() >= 0, expert_out.cpu().double()[places.clamp(min=0).long().cpu()].view(tokens, top, width),
+                         h.cpu().double()[:, None, :].expand(tokens, top, width))
+    branch = (weights.cpu().double()[:, :, None] * picked).sum(dim=1)
+    unit = lambda x: x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5)
+    want = stream.cpu().double() + 0.4 * unit(branch) * w_branch.cpu().double()
+    assert torch.allclose(a.cpu().double(), want, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(rows_a.cpu().double(), unit(want) * w_next.cpu().double(), rtol=2e-2 if dtype == torch.bfloat16 else 1e-5, atol=1e-2 if dtype == torch.bfloat16 else 1e-5)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     folder = folders("A", stored_as(dtype))
